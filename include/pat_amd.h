@@ -1,0 +1,230 @@
+/*
+ * pat_amd.h — C ABI of libpat_amd: prefix-aware decode attention over a paged KV
+ * cache for AMD MI355X (gfx950).
+ *
+ * Everything here is plain C: integers, pointers and sizes. No torch / pybind types.
+ * A binding (ctypes, pybind11, cgo ...) converts its tensors to raw pointers +
+ * element strides and calls these entry points.
+ *
+ * Every function returns PAT_OK (0) or a negative PAT_ERR_* code; the message of
+ * the last failure on the calling thread is returned by pat_last_error().
+ *
+ * Reference interfaces replaced (paths relative to the flashserve/PAT tree):
+ *   scheduler        prefix_attn/prefix_tree.py:47-616  (class PrefixTree)
+ *                    csrc/prefix_tree.h:63-324          (PrefixTreeCPP twin)
+ *                    csrc/bindings.cpp:100-146          (its pybind surface)
+ *   plan containers  prefix_attn/data_class.py:173-254  (KernelInfo / to_tensor)
+ *   forward          csrc/api.h:110-295                 (pat_mha_fwd_kvcache)
+ *                    csrc/bindings.cpp:7-72             (both Python overloads)
+ *   kernels          csrc/pat_fwd_kernel.h:25-310       (split-KV forward)
+ *                    csrc/pat_fwd_kernel.h:314-467      (gather / merge)
+ *                    csrc/pat_fwd_launch_template.h:35-98 (dispatch)
+ */
+#ifndef PAT_AMD_H_
+#define PAT_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PAT_ABI_VERSION 1
+
+/* ---- status codes ------------------------------------------------------- */
+#define PAT_OK 0
+#define PAT_ERR_INVALID (-1) /* bad argument; bindings raise RuntimeError          */
+#define PAT_ERR_VALUE (-2)   /* where the Python scheduler raises ValueError        */
+#define PAT_ERR_INDEX (-3)   /* where the Python scheduler raises IndexError        */
+#define PAT_ERR_KEY (-4)     /* where the Python scheduler raises KeyError          */
+#define PAT_ERR_HIP (-5)     /* a HIP runtime call failed                           */
+#define PAT_ERR_WORKSPACE (-6) /* workspace missing or too small                    */
+
+#define PAT_DTYPE_F16 0
+#define PAT_DTYPE_BF16 1
+
+/* Message of the last error raised on this thread ("" if none). Never NULL. */
+const char* pat_last_error(void);
+/* Returns PAT_ABI_VERSION of the loaded library. */
+int pat_abi_version(void);
+
+/* ======================================================================== *
+ *  Scheduler: radix tree over block-table rows -> packed boxes -> buckets   *
+ * ======================================================================== */
+
+typedef struct pat_tree pat_tree; /* opaque */
+
+/* Tuning constants of the load balancer. Passing NULL to pat_tree_pack keeps the
+ * reference's values (prefix_attn/prefix_tree.py:390-437), which is what plan
+ * parity is defined against. */
+typedef struct pat_sched_opts {
+  int32_t long_kv_tokens;      /* boxes with kv > this enter the average (256)        */
+  int32_t long_factor;         /* a box is cut when blocks > factor * average (5)      */
+  int32_t min_boxes[5];        /* target #boxes for kv_heads <=4,<=8,<=16,<=32,else    */
+                               /* (54, 27, 13, 6, 4)                                   */
+  int32_t stop_blocks;         /* halving stops at boxes of <= this many blocks (8)    */
+  int32_t max_split;           /* halving stops once a sequence has this many (32)     */
+} pat_sched_opts;
+
+/* One node of the radix tree (for inspection / tests). Pointers alias tree storage
+ * and stay valid until the tree is rebuilt or destroyed. */
+typedef struct pat_node_view {
+  int32_t parent;       /* -1 for the root                                   */
+  int32_t num_seqs;     /* s_value: sequences passing through the node       */
+  int32_t num_tokens;   /* tokens of KV held by the node                     */
+  int32_t num_seq_ids;  /* length of seq_ids                                 */
+  int32_t num_blocks;   /* length of block_ids                               */
+  int32_t num_children; /* length of child_ids (insertion order)             */
+  const int32_t* seq_ids;
+  const int32_t* block_ids;
+  const int32_t* child_ids;
+} pat_node_view;
+
+/* One tile bucket of a plan. Rows of q_table / block_table are padded with 0 to
+ * the bucket's widest row, exactly as KernelInfo.to_tensor does
+ * (prefix_attn/data_class.py:228-253). q_len / block_len keep the unpadded
+ * lengths so a binding can also rebuild the ragged Python lists. */
+typedef struct pat_bucket_view {
+  int32_t mnw[3];       /* tile label [M, N, W] of the bucket                */
+  int32_t num_boxes;    /* "CTAs" in the reference                            */
+  int32_t max_seqs;     /* q_table row width                                  */
+  int32_t max_blocks;   /* block_table row width                              */
+  const int32_t* q_table;     /* [num_boxes, max_seqs]                        */
+  const int32_t* block_table; /* [num_boxes, max_blocks]                      */
+  const int32_t* q_len;       /* [num_boxes]                                  */
+  const int32_t* block_len;   /* [num_boxes]                                  */
+  const int32_t* num_seqs;    /* [num_boxes]  num_seqs_per_CTA                */
+  const int32_t* rank;        /* [num_boxes]  CTA_rank                        */
+  const int32_t* kv;          /* [num_boxes]  kv_in_CTA (tokens)              */
+} pat_bucket_view;
+
+typedef struct pat_plan_view {
+  int32_t num_buckets;
+  int32_t batch;                    /* length of num_split_per_seq            */
+  const pat_bucket_view* buckets;   /* [num_buckets]                          */
+  const int32_t* num_split_per_seq; /* [batch]                                */
+  int32_t max_split_per_seq;
+  int32_t max_seqs_in_box;          /* KernelInfo.max_seqs_in_CTA             */
+  int32_t max_blocks_in_box;        /* KernelInfo.max_blocks_in_CTA           */
+} pat_plan_view;
+
+/* PrefixTree(block_size)                     prefix_attn/prefix_tree.py:48-59 */
+int pat_tree_create(int32_t block_size, pat_tree** out);
+void pat_tree_destroy(pat_tree* tree);
+
+/* PrefixTreeCPP.build_radix_tree(seq_lens, block_table)
+ *                                  csrc/bindings.cpp:103-126, prefix_tree.h:84-99
+ * table is a dense [num_seqs, max_blocks] matrix; row i contributes its first
+ * ceil(seq_lens[i] / block_size) entries, the rest is padding. The table is copied:
+ * the caller may free it as soon as the call returns. */
+int pat_tree_build(pat_tree* tree, const int32_t* seq_lens, const int32_t* table,
+                   int32_t num_seqs, int32_t max_blocks);
+
+/* PrefixTree.build_radix_tree(seq_lens, block_table: List[List[int]])
+ *                                             prefix_attn/prefix_tree.py:146-149
+ * Ragged rows: row i is flat_blocks[row_offsets[i] .. row_offsets[i+1]) and is used
+ * whole, whatever seq_lens[i] says (as the Python class does). */
+int pat_tree_build_rows(pat_tree* tree, const int32_t* seq_lens,
+                        const int32_t* flat_blocks, const int64_t* row_offsets,
+                        int32_t num_seqs);
+
+/* PrefixTree.pack_schedule(MNWs, HRatio, kvHead, use_compute_model)
+ *                                             prefix_attn/prefix_tree.py:548-616
+ * mnws: n_mnws triples [M, N, W] or NULL (n_mnws 0) for the default 11 buckets.
+ * The resulting plan is stored in the tree; read it with pat_tree_plan. As in the
+ * Python class, the per-sequence split counters are NOT reset between calls. */
+int pat_tree_pack(pat_tree* tree, const int32_t* mnws, int32_t n_mnws, int32_t hratio,
+                  int32_t kv_heads, int32_t use_compute_model,
+                  const pat_sched_opts* opts);
+
+/* PrefixTree.naive_schedule(HRatio)           prefix_attn/prefix_tree.py:484-545 */
+int pat_tree_naive_schedule(pat_tree* tree, int32_t hratio);
+
+/* Borrow the plan built by the last pack / naive_schedule call. */
+int pat_tree_plan(const pat_tree* tree, pat_plan_view* out);
+
+int pat_tree_num_nodes(const pat_tree* tree);
+int pat_tree_node(const pat_tree* tree, int32_t node, pat_node_view* out);
+
+/* ======================================================================== *
+ *  Forward: split-KV kernels over the plan + LSE merge                      *
+ * ======================================================================== */
+
+/* Per-bucket plan tables, resident in device memory (int32). */
+typedef struct pat_fwd_bucket {
+  const int32_t* q_table;     /* [num_boxes, q_table_stride]                  */
+  const int32_t* block_table; /* [num_boxes, block_table_stride]              */
+  const int32_t* num_seqs;    /* [num_boxes]                                  */
+  const int32_t* rank;        /* [num_boxes]                                  */
+  const int32_t* kv;          /* [num_boxes]                                  */
+  int64_t q_table_stride;     /* elements between rows                        */
+  int64_t block_table_stride; /* elements between rows                        */
+  int32_t num_boxes;
+  int32_t max_seqs;           /* valid columns of q_table                     */
+  int32_t max_blocks;         /* valid columns of block_table                 */
+  int32_t mnw[3];
+} pat_fwd_bucket;
+
+/* Mirrors the arguments of pat_mha_fwd_kvcache (csrc/api.h:110-127).
+ * Strides are in ELEMENTS (as csrc/api.h:43); the last dimension of q, k, v, out
+ * must be contiguous. Unlike the reference, V may have strides of its own. */
+typedef struct pat_fwd_args {
+  int32_t dtype;       /* PAT_DTYPE_F16 | PAT_DTYPE_BF16 (q, k, v, out)      */
+  int32_t batch;       /* q.size(0)                                           */
+  int32_t seqlen_q;    /* q.size(1); decode: 1                                */
+  int32_t heads;       /* q.size(2)                                           */
+  int32_t kv_heads;    /* k.size(2)                                           */
+  int32_t head_dim;    /* 64 | 128                                            */
+  int32_t page_size;   /* k.size(1), multiple of 16                           */
+  int32_t num_pages;   /* k.size(0)                                           */
+  const void* q;       /* [batch, 1, heads, head_dim]                         */
+  const void* k;       /* [num_pages, page_size, kv_heads, head_dim]          */
+  const void* v;
+  void* out;           /* [batch, 1, heads, head_dim], written in place       */
+  float* lse_out;      /* optional [batch, heads] natural-log LSE, or NULL    */
+  int64_t q_stride[3]; /* batch, row, head                                    */
+  int64_t k_stride[3]; /* page, slot, head                                    */
+  int64_t v_stride[3];
+  int64_t o_stride[3]; /* batch, row, head                                    */
+  const int32_t* num_split_per_seq; /* device int32 [batch]                   */
+  int32_t max_split_per_seq;
+  int32_t max_seqs_in_box;
+  int32_t max_blocks_in_box;
+  float softmax_scale;
+  int32_t num_buckets;
+  const pat_fwd_bucket* buckets; /* host array [num_buckets]                  */
+  void* workspace;               /* device scratch, 256-byte aligned          */
+  size_t workspace_bytes;
+} pat_fwd_args;
+
+/* Argument checks of csrc/api.h:129-181 that need no GPU (dtype enum, head_dim,
+ * page size, GQA ratio, split limits, strides, bucket labels). Pointers are only
+ * tested for NULL. Runs on a machine without a GPU. */
+int pat_fwd_validate(const pat_fwd_args* args);
+
+/* Bytes of device scratch pat_fwd_launch needs for these arguments (partial
+ * outputs + partial LSE; the reference allocates the equivalent per call at
+ * csrc/api.h:217-229). Depends only on sizes, never on device data. */
+int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
+
+/* prefix_attn_with_kvcache(...)   csrc/bindings.cpp:7-72 -> csrc/api.h:110-295
+ * Enqueues the split-KV kernels and the merge kernel on `hip_stream`
+ * (a hipStream_t; NULL = the null stream) of the current device and returns
+ * without synchronising. */
+int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
+
+/* Description of the launch geometry chosen for `args` (for benchmarks/tests). */
+typedef struct pat_fwd_geometry {
+  int32_t chunk_tokens;     /* KV tokens one workgroup streams                */
+  int32_t chunks_per_rank;  /* partial slots reserved per CTA_rank            */
+  int32_t num_slots;        /* max_split_per_seq * chunks_per_rank            */
+  int32_t num_launches;     /* split-kernel launches (one per row-tile class) */
+  int64_t num_workgroups;   /* total split-kernel workgroups                  */
+} pat_fwd_geometry;
+int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* PAT_AMD_H_ */

@@ -1,0 +1,277 @@
+"""The extension-module surface of the reference (`prefix_attn._prefix_attn`), served by
+libpat_amd through its C ABI.
+
+Mirrors csrc/bindings.cpp of the flashserve/PAT tree:
+  * `prefix_attn_with_kvcache` — table overload (:7-43, :76-95) and tree overload
+    (:45-72, :148-157), told apart by the 4th argument;
+  * `PrefixTreeCPP` (:100-146) with `build_radix_tree`, `pack_schedule`, `kernel_info`;
+  * `KernelInfo.to_gpu(device)` (:97-98).
+torch is used for what a binding needs from it: data pointers, strides, the current
+HIP stream and scratch memory from the caching allocator. All computation happens in
+the HIP kernels of libpat_amd; there is no PyTorch fallback path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from . import _lib
+from .prefix_tree import _NativeTree
+
+__all__ = ["prefix_attn_with_kvcache", "PrefixTreeCPP", "KernelInfo"]
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+class KernelInfo:
+    """Plan tensors of a `PrefixTreeCPP`: int32, on the CPU after `pack_schedule`, moved to
+    the GPU by `to_gpu` (csrc/prefix_tree.h:7-39)."""
+
+    def __init__(self) -> None:
+        self.q_tables: List[torch.Tensor] = []
+        self.block_tables: List[torch.Tensor] = []
+        self.num_seqs_per_CTAs: List[torch.Tensor] = []
+        self.CTA_ranks: List[torch.Tensor] = []
+        self.kv_in_CTAs: List[torch.Tensor] = []
+        self.MNWs: List[List[int]] = []
+        self.num_split_per_seq: torch.Tensor = torch.empty(0, dtype=torch.int32)
+        self.max_split_per_seq = 0
+        self.max_seqs_in_CTA = 0
+        self.max_blocks_in_CTA = 0
+        self._launch_cache: dict = {}
+
+    def to_gpu(self, device: Union[torch.device, str]) -> None:
+        """Copies every plan tensor to `device` (asynchronously where the source is pinned)."""
+        device = torch.device(device)
+
+        def move(t: torch.Tensor) -> torch.Tensor:
+            return t.to(device, non_blocking=True)
+
+        self.q_tables = [move(t) for t in self.q_tables]
+        self.block_tables = [move(t) for t in self.block_tables]
+        self.num_seqs_per_CTAs = [move(t) for t in self.num_seqs_per_CTAs]
+        self.CTA_ranks = [move(t) for t in self.CTA_ranks]
+        self.kv_in_CTAs = [move(t) for t in self.kv_in_CTAs]
+        self.num_split_per_seq = move(self.num_split_per_seq)
+        self._launch_cache.clear()
+
+    @classmethod
+    def _from_view(cls, view: _lib.PlanView) -> "KernelInfo":
+        ki = cls()
+        for b in range(view.num_buckets):
+            bk = view.buckets[b]
+            n, ws, wb = bk.num_boxes, bk.max_seqs, bk.max_blocks
+
+            def mat(ptr, w):
+                a = np.ctypeslib.as_array(ptr, shape=(n, w)) if w else np.zeros((n, 0), np.int32)
+                return torch.from_numpy(a.copy())
+
+            def vec(ptr):
+                return torch.from_numpy(np.ctypeslib.as_array(ptr, shape=(n,)).copy())
+
+            ki.MNWs.append([bk.mnw[0], bk.mnw[1], bk.mnw[2]])
+            ki.q_tables.append(mat(bk.q_table, ws))
+            ki.block_tables.append(mat(bk.block_table, wb))
+            ki.num_seqs_per_CTAs.append(vec(bk.num_seqs))
+            ki.CTA_ranks.append(vec(bk.rank))
+            ki.kv_in_CTAs.append(vec(bk.kv))
+        ki.num_split_per_seq = torch.from_numpy(
+            np.ctypeslib.as_array(view.num_split_per_seq, shape=(view.batch,)).copy())
+        ki.max_split_per_seq = view.max_split_per_seq
+        ki.max_seqs_in_CTA = view.max_seqs_in_box
+        ki.max_blocks_in_CTA = view.max_blocks_in_box
+        return ki
+
+
+class PrefixTreeCPP:
+    """Native radix tree + scheduler over a padded block table.
+
+    `build_radix_tree(seq_lens, block_table)`: `seq_lens` is a list of ints or a CPU int32
+    tensor, `block_table` a contiguous CPU int32 tensor [num_seqs, max_blocks]; row i uses
+    its first ceil(seq_lens[i] / block_size) entries. `pack_schedule` stores the plan in
+    `kernel_info`. Both release the GIL while the native code runs.
+    """
+
+    def __init__(self, block_size: int):
+        self.block_size = int(block_size)
+        self._native = _NativeTree(self.block_size)
+        self.kernel_info = KernelInfo()
+
+    def build_radix_tree(self, seq_lens: Union[List[int], torch.Tensor], block_table: torch.Tensor) -> None:
+        _check(isinstance(block_table, torch.Tensor) and block_table.dim() == 2,
+               "block_table must be a 2-D CPU Int32 Tensor")
+        _check(block_table.device.type == "cpu" and block_table.dtype == torch.int32,
+               "block_table must be a CPU Int32 Tensor")
+        table = np.ascontiguousarray(block_table.numpy())
+        if isinstance(seq_lens, torch.Tensor):
+            _check(seq_lens.device.type == "cpu" and seq_lens.dtype == torch.int32,
+                   "seq_lens must be a List[int] or a CPU Int32 Tensor")
+            lens = np.ascontiguousarray(seq_lens.numpy().reshape(-1))
+        elif isinstance(seq_lens, list):
+            lens = np.asarray(seq_lens, dtype=np.int32)
+        else:
+            raise RuntimeError("seq_lens must be a List[int] or a CPU Int32 Tensor")
+        _check(lens.shape[0] == table.shape[0], "Seq lens list mismatch")
+        self._native.build_table(lens, table)
+
+    def pack_schedule(self, MNWs: Optional[List[List[int]]] = None, HRatio: int = 1, kvHead: int = 8,
+                      use_compute_model: bool = False) -> None:
+        if MNWs is not None and len(MNWs) == 0:
+            MNWs = None  # an empty list selects the default buckets (csrc/prefix_tree.h:189)
+        self._native.pack(MNWs, HRatio, kvHead, use_compute_model)
+        self.kernel_info = KernelInfo._from_view(self._native.plan_view())
+
+
+# --------------------------------------------------------------------------------------
+#  forward
+# --------------------------------------------------------------------------------------
+
+def _strides3(t: torch.Tensor):
+    return (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+class _Launch:
+    """A prepared pat_fwd_args (+ the tensors it points into, kept alive)."""
+    __slots__ = ("args", "buckets", "keep", "workspace", "need")
+
+
+def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MNW, max_split,
+             max_seqs, max_blocks, scale, out, lse) -> _Launch:
+    lib = _lib.load()
+    # --- checks that need tensor metadata (csrc/api.h:131-181, :256-277) -----------------
+    _check(q.dtype in (torch.float16, torch.bfloat16), "only support fp16 and bf16 data type")
+    _check(k.dtype == q.dtype, "query and key must have the same dtype")
+    _check(v.dtype == q.dtype, "query and value must have the same dtype")
+    for name, t in (("q", q), ("kcache", k), ("vcache", v)):
+        _check(t.is_cuda, f"{name} must be on CUDA")
+    for t in (q, k, v):
+        _check(t.dim() == 4 and t.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    b, sq, h, d = q.shape
+    nblk, page, hk, dk = k.shape
+    _check(tuple(k.shape) == (nblk, page, hk, d), "kcache must have shape (num_blocks, page_block_size, n_heads_kv, head_size_og)")
+    _check(tuple(v.shape) == (nblk, page, hk, d), "vcache must have shape (num_blocks, page_block_size, n_heads_kv, head_size_og)")
+    _check(out.is_cuda and out.dtype == q.dtype and tuple(out.shape) == tuple(q.shape) and out.stride(-1) == 1,
+           "out must be a CUDA tensor with q's shape and dtype and a contiguous last dimension")
+    _check(num_split.is_cuda, "num_split_per_seq must be on CUDA")
+    _check(num_split.dtype == torch.int32, "num_split_per_seq must have dtype torch.int32")
+    _check(num_split.stride(-1) == 1, "num_split_per_seq must have contiguous last dimension")
+    _check(tuple(num_split.shape) == (b,), "num_split_per_seq must have shape (batch_size)")
+    nb = len(MNW)
+    _check(all(len(x) == nb for x in (q_tables, block_tables, num_seqs, ranks, kvs)),
+           "MNW and the per-bucket plan lists must have the same length")
+
+    L = _Launch()
+    L.buckets = (_lib.FwdBucket * max(nb, 1))()
+    for i in range(nb):
+        qt, bt, ns, rk, kv = q_tables[i], block_tables[i], num_seqs[i], ranks[i], kvs[i]
+        ctas = qt.shape[0]
+        for name, t in (("query_tables", qt), ("block_tables", bt), ("num_seqs_per_CTA", ns),
+                        ("CTA_rank", rk), ("kv_in_CTA", kv)):
+            _check(t.is_cuda, f"{name} must be on CUDA")
+            _check(t.dtype == torch.int32, f"{name} must have dtype torch.int32")
+            _check(t.numel() == 0 or t.stride(-1) == 1, f"{name} must have contiguous last dimension")
+        _check(qt.dim() == 2 and bt.dim() == 2 and bt.shape[0] == ctas, "query_tables / block_tables must be (CTAs, width)")
+        for name, t in (("num_seqs_per_CTA", ns), ("CTA_rank", rk), ("kv_in_CTA", kv)):
+            _check(tuple(t.shape) == (ctas,), f"{name} must have shape (CTAs)")
+        fb = L.buckets[i]
+        fb.q_table, fb.block_table = qt.data_ptr(), bt.data_ptr()
+        fb.num_seqs, fb.rank, fb.kv = ns.data_ptr(), rk.data_ptr(), kv.data_ptr()
+        fb.q_table_stride = qt.stride(0) if ctas > 1 else max(qt.shape[1], 1)
+        fb.block_table_stride = bt.stride(0) if ctas > 1 else max(bt.shape[1], 1)
+        fb.num_boxes, fb.max_seqs, fb.max_blocks = ctas, qt.shape[1], bt.shape[1]
+        fb.mnw[0], fb.mnw[1], fb.mnw[2] = int(MNW[i][0]), int(MNW[i][1]), int(MNW[i][2])
+
+    a = _lib.FwdArgs()
+    a.dtype = _lib.PAT_DTYPE_BF16 if q.dtype == torch.bfloat16 else _lib.PAT_DTYPE_F16
+    a.batch, a.seqlen_q, a.heads, a.kv_heads = b, sq, h, hk
+    a.head_dim, a.page_size, a.num_pages = d, page, nblk
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_stride, a.k_stride, a.v_stride, a.o_stride = _strides3(q), _strides3(k), _strides3(v), _strides3(out)
+    a.num_split_per_seq = num_split.data_ptr()
+    a.max_split_per_seq, a.max_seqs_in_box, a.max_blocks_in_box = int(max_split), int(max_seqs), int(max_blocks)
+    a.softmax_scale = float(scale)
+    a.num_buckets = nb
+    a.buckets = C.cast(L.buckets, C.POINTER(_lib.FwdBucket))
+    if lse is not None:
+        _check(lse.is_cuda and lse.dtype == torch.float32 and lse.is_contiguous() and lse.numel() == b * h,
+               "softmax_lse must be a contiguous CUDA float32 tensor with batch_size * n_heads elements")
+        a.lse_out = lse.data_ptr()
+    need = C.c_size_t(0)
+    _lib.check(lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)))
+    L.args, L.need = a, need.value
+    # plan tensors stay referenced as long as the prepared launch does; q/k/v/out are the
+    # caller's for the duration of the call only
+    L.keep = (num_split, list(q_tables), list(block_tables), list(num_seqs), list(ranks), list(kvs))
+    L.workspace = None
+    return L
+
+
+def _run(L: _Launch, device: torch.device) -> None:
+    lib = _lib.load()
+    # scratch for the partial results, from torch's caching allocator on the current stream
+    ws = torch.empty(L.need, dtype=torch.uint8, device=device)
+    L.args.workspace = ws.data_ptr()
+    L.args.workspace_bytes = L.need
+    stream = torch.cuda.current_stream(device).cuda_stream
+    _lib.check(lib.pat_fwd_launch(C.byref(L.args), C.c_void_p(stream)))
+
+
+def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cache_paged: torch.Tensor,
+                             *rest, **kw) -> None:
+    """Prefix-aware decode attention over a paged KV cache; writes `out` in place.
+
+    Table form:  (q, k_cache_paged, v_cache_paged, num_split_per_seq, query_tables, block_tables,
+                  num_seqs_per_CTAs, CTA_ranks, kv_in_CTAs, MNW, max_split_per_seq, max_seqs_in_CTA,
+                  max_blocks_in_CTA, softmax_scale, out, timing_=None)
+    Tree form:   (q, k_cache_paged, v_cache_paged, tree, softmax_scale, out)
+    Both accept the extra keyword `softmax_lse` (float32 [batch, heads]) to receive the
+    natural-log LSE, which the reference computes but does not return.
+    """
+    lse = kw.pop("softmax_lse", None)
+    tree_names = ("tree", "softmax_scale", "out")
+    table_names = ("num_split_per_seq", "query_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks",
+                   "kv_in_CTAs", "MNW", "max_split_per_seq", "max_seqs_in_CTA", "max_blocks_in_CTA",
+                   "softmax_scale", "out", "timing_")
+    is_tree = "tree" in kw or (len(rest) > 0 and isinstance(rest[0], PrefixTreeCPP))
+    names = tree_names if is_tree else table_names
+    if len(rest) > len(names):
+        raise TypeError("prefix_attn_with_kvcache(): incompatible function arguments")
+    vals = dict(zip(names, rest))
+    for key, val in kw.items():
+        if key not in names or key in vals:
+            raise TypeError(f"prefix_attn_with_kvcache(): incompatible function arguments ({key})")
+        vals[key] = val
+    missing = [nm for nm in names if nm not in vals and nm != "timing_"]
+    if missing:
+        raise TypeError(f"prefix_attn_with_kvcache(): missing arguments {missing}")
+
+    out = vals["out"]
+    with torch.cuda.device(q.device):
+        if is_tree:
+            tree = vals["tree"]
+            tree = getattr(tree, "tree", tree) if not isinstance(tree, PrefixTreeCPP) else tree
+            info = tree.kernel_info
+            key = (q.data_ptr(), k_cache_paged.data_ptr(), v_cache_paged.data_ptr(), out.data_ptr(),
+                   tuple(q.shape), q.stride(), k_cache_paged.stride(), v_cache_paged.stride(), out.stride(),
+                   q.dtype, float(vals["softmax_scale"]), None if lse is None else lse.data_ptr())
+            L = info._launch_cache.get(key)
+            if L is None:
+                L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, info.q_tables,
+                             info.block_tables, info.num_seqs_per_CTAs, info.CTA_ranks, info.kv_in_CTAs,
+                             info.MNWs, info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                             vals["softmax_scale"], out, lse)
+                if len(info._launch_cache) >= 256:
+                    info._launch_cache.clear()
+                info._launch_cache[key] = L
+        else:
+            L = _prepare(q, k_cache_paged, v_cache_paged, vals["num_split_per_seq"], vals["query_tables"],
+                         vals["block_tables"], vals["num_seqs_per_CTAs"], vals["CTA_ranks"], vals["kv_in_CTAs"],
+                         vals["MNW"], vals["max_split_per_seq"], vals["max_seqs_in_CTA"],
+                         vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse)
+        _run(L, q.device)

@@ -1,0 +1,261 @@
+// extern "C" forward entry points (declared in include/pat_amd.h): argument checks,
+// launch geometry, workspace sizing and kernel launches. Host code only; the kernels
+// live in hip/pat_split.hip and hip/pat_merge.hip.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+#include "capi_error.hpp"
+#include "hip/fwd_params.hpp"
+#include "pat_amd.h"
+
+namespace pat {
+
+// defined next to the kernels (hip/pat_split.hip, hip/pat_merge.hip)
+hipError_t launch_split(bool bf16, int head_dim, int row_tiles, unsigned workgroups, hipStream_t stream,
+                        const SplitParams& params);
+hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params);
+
+namespace {
+
+constexpr int kNumCUs = 256;        // MI355X
+constexpr int kMaxChunksPerRank = 64;
+
+inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
+
+// Row-tile class of a bucket from its tile label: M in {16, 32, 64} -> 1, 2, 4 tiles
+// of 16 rows. The label is only that here: a size class (the kernels pick their own
+// tiling), so page size never restricts which label is usable (the reference refuses
+// (16,128,1) for pages under 32 tokens, csrc/api.h:177-181).
+inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 2 : 4); }
+
+struct Geometry {
+  int chunk = 0;             // tokens per workgroup
+  int chunks_per_rank = 0;   // widest bucket's chunk count
+  int num_slots = 0;
+  int bucket_chunks[kMaxBuckets] = {0};
+  int64_t class_wgs[3] = {0, 0, 0};  // workgroups per row-tile class (1, 2, 4 tiles)
+  int64_t total_wgs = 0;
+  int launches = 0;
+};
+
+int check_args(const pat_fwd_args* a) {
+  if (a == nullptr) return fail(PAT_ERR_INVALID, "args is NULL");
+  // messages follow csrc/api.h:131-181 of the reference where a counterpart exists
+  if (a->dtype != PAT_DTYPE_F16 && a->dtype != PAT_DTYPE_BF16)
+    return fail(PAT_ERR_INVALID, "only support fp16 and bf16 data type");
+  if (a->q == nullptr || a->k == nullptr || a->v == nullptr || a->out == nullptr)
+    return fail(PAT_ERR_INVALID, "q, k_cache_paged, v_cache_paged and out must be non-null device tensors");
+  if (a->max_split_per_seq > 32)
+    return fail(PAT_ERR_INVALID,
+                "Currently, only supports up to 32 splits per seq. Excessive splitting may reduce efficiency.");
+  if (a->max_split_per_seq <= 0)
+    return fail(PAT_ERR_INVALID, "there is no case that a seq has no block");
+  if (a->head_dim != 64 && a->head_dim != 128)
+    return fail(PAT_ERR_INVALID, "head_size_og must be 64 / 128 currently");
+  if (a->page_size <= 0 || a->page_size % 16 != 0)
+    return fail(PAT_ERR_INVALID, "Paged KV cache block size must be divisible by 16");
+  if (a->kv_heads <= 0 || a->heads <= 0 || a->heads % a->kv_heads != 0)
+    return fail(PAT_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
+  const int ratio = a->heads / a->kv_heads;
+  if (ratio != 1 && ratio != 2 && ratio != 4 && ratio != 8)
+    return fail(PAT_ERR_INVALID, "only support QGA with hq/hkv = 1, 2, 4, 8 now.");
+  if (a->batch <= 0) return fail(PAT_ERR_INVALID, "batch size must be positive");
+  if (a->seqlen_q != 1) return fail(PAT_ERR_INVALID, "q must have shape (batch_size, 1, n_heads, head_size): decode only");
+  if (a->num_pages <= 0) return fail(PAT_ERR_INVALID, "k_cache_paged must hold at least one block");
+  if (a->num_split_per_seq == nullptr)
+    return fail(PAT_ERR_INVALID, "num_split_per_seq must be a device int32 tensor of shape (batch_size)");
+  // 16-byte vector loads: rows of q/k/v must start on 16-byte boundaries
+  const int64_t* strides[3] = {a->q_stride, a->k_stride, a->v_stride};
+  const char* names[3] = {"q", "k_cache_paged", "v_cache_paged"};
+  for (int t = 0; t < 3; ++t)
+    for (int i = 0; i < 3; ++i)
+      if (strides[t][i] % 8 != 0 || strides[t][i] < 0)
+        return fail(PAT_ERR_INVALID, std::string(names[t]) + " strides must be non-negative multiples of 8 elements");
+  const void* ptrs[3] = {a->q, a->k, a->v};
+  for (int t = 0; t < 3; ++t)
+    if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0)
+      return fail(PAT_ERR_INVALID, std::string(names[t]) + " must be 16-byte aligned");
+  if (a->o_stride[0] < 0 || a->o_stride[2] < 0)
+    return fail(PAT_ERR_INVALID, "out strides must be non-negative");
+  if (a->num_buckets <= 0 || a->num_buckets > kMaxBuckets || a->buckets == nullptr)
+    return fail(PAT_ERR_INVALID, "MNW must list between 1 and 12 tile buckets");
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const pat_fwd_bucket& b = a->buckets[i];
+    const std::string at = " (bucket " + std::to_string(i) + ")";
+    if (b.mnw[0] != 16 && b.mnw[0] != 32 && b.mnw[0] != 64)
+      return fail(PAT_ERR_INVALID, "MNW tile_q must be 16, 32 or 64" + at);
+    if (b.num_boxes < 0 || b.max_seqs < 0 || b.max_blocks < 0)
+      return fail(PAT_ERR_INVALID, "plan table sizes must be non-negative" + at);
+    if (b.num_boxes > 0 && (b.q_table == nullptr || b.block_table == nullptr || b.num_seqs == nullptr ||
+                            b.rank == nullptr || b.kv == nullptr))
+      return fail(PAT_ERR_INVALID, "plan tables must be device int32 tensors" + at);
+    if (b.q_table_stride < b.max_seqs || b.block_table_stride < b.max_blocks)
+      return fail(PAT_ERR_INVALID, "plan table row stride smaller than its width" + at);
+    if (b.q_table_stride > INT32_MAX || b.block_table_stride > INT32_MAX)
+      return fail(PAT_ERR_INVALID, "plan table row stride too large" + at);
+    if ((int64_t)b.max_seqs * ratio > 64)
+      return fail(PAT_ERR_INVALID, "a box may pack at most 64 rows (sequences x heads per kv head)" + at);
+  }
+  return PAT_OK;
+}
+
+// Launch geometry: one chunk size for the whole call. Sized so the device sees a few
+// workgroups per CU; a bucket reserves ceil(widest box / chunk) workgroups per box.
+int plan_geometry(const pat_fwd_args* a, Geometry* g) {
+  const int page = a->page_size;
+  const int64_t unit = (int64_t)page * kStepTokens / gcd64(page, kStepTokens);  // lcm(page, 32)
+  int64_t total = 0, widest = 0;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+    total += tok * a->buckets[i].num_boxes * a->kv_heads;
+    widest = std::max(widest, tok);
+  }
+  int64_t chunk = 0;
+  if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
+  if (chunk <= 0) {
+    // aim at ~4 workgroups per CU, between 128 and 1024 tokens each
+    chunk = total / (4 * kNumCUs);
+    chunk = std::max<int64_t>(128, std::min<int64_t>(1024, chunk));
+  }
+  chunk = std::max<int64_t>(unit, ceil_div64(chunk, unit) * unit);
+  // bounded slot count per rank, and page ids of a chunk must fit their LDS table
+  while (ceil_div64(widest, chunk) > kMaxChunksPerRank) chunk += unit;
+  if (chunk / page > kMaxChunkPages) {
+    chunk = (int64_t)kMaxChunkPages * page / unit * unit;
+    if (chunk <= 0 || ceil_div64(widest, chunk) > kMaxChunksPerRank)
+      return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
+  }
+  g->chunk = (int)chunk;
+  g->chunks_per_rank = 1;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+    const int c = (int)std::max<int64_t>(1, ceil_div64(tok, chunk));
+    g->bucket_chunks[i] = c;
+    g->chunks_per_rank = std::max(g->chunks_per_rank, c);
+    const int cls = row_tiles(a->buckets[i].mnw[0]) >> 1;  // 1,2,4 -> 0,1,2
+    g->class_wgs[cls] += (int64_t)a->buckets[i].num_boxes * c * a->kv_heads;
+  }
+  g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
+  g->total_wgs = 0;
+  g->launches = 0;
+  for (int c = 0; c < 3; ++c) {
+    if (g->class_wgs[c] > INT32_MAX) return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
+    g->total_wgs += g->class_wgs[c];
+    g->launches += g->class_wgs[c] > 0;
+  }
+  return PAT_OK;
+}
+
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t workspace_need(const pat_fwd_args* a, const Geometry& g) {
+  const size_t rows = (size_t)a->batch * a->heads * g.num_slots;
+  return align256(rows * a->head_dim * sizeof(float)) + align256(rows * sizeof(float));
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(PAT_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+}  // namespace
+}  // namespace pat
+
+extern "C" {
+
+int pat_fwd_validate(const pat_fwd_args* args) { return pat::check_args(args); }
+
+int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out) {
+  if (out == nullptr) return pat::fail(PAT_ERR_INVALID, "out is NULL");
+  if (int rc = pat::check_args(args)) return rc;
+  pat::Geometry g;
+  if (int rc = pat::plan_geometry(args, &g)) return rc;
+  out->chunk_tokens = g.chunk;
+  out->chunks_per_rank = g.chunks_per_rank;
+  out->num_slots = g.num_slots;
+  out->num_launches = g.launches;
+  out->num_workgroups = g.total_wgs;
+  return PAT_OK;
+}
+
+int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes) {
+  if (bytes == nullptr) return pat::fail(PAT_ERR_INVALID, "bytes is NULL");
+  if (int rc = pat::check_args(args)) return rc;
+  pat::Geometry g;
+  if (int rc = pat::plan_geometry(args, &g)) return rc;
+  *bytes = pat::workspace_need(args, g);
+  return PAT_OK;
+}
+
+int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
+  using namespace pat;
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  const size_t need = workspace_need(args, g);
+  if (args->workspace == nullptr || args->workspace_bytes < need)
+    return fail(PAT_ERR_WORKSPACE, "workspace too small: need " + std::to_string(need) + " bytes, got " +
+                                       std::to_string(args->workspace_bytes));
+  if (reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
+    return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+
+  const size_t rows = (size_t)args->batch * args->heads * g.num_slots;
+  float* o_part = static_cast<float*>(args->workspace);
+  float* lse_part = reinterpret_cast<float*>(static_cast<char*>(args->workspace) +
+                                             align256(rows * args->head_dim * sizeof(float)));
+
+  SplitParams sp;
+  std::memset(&sp, 0, sizeof(sp));
+  sp.q = args->q; sp.k = args->k; sp.v = args->v;
+  sp.o_part = o_part; sp.lse_part = lse_part;
+  sp.q_stride_b = args->q_stride[0]; sp.q_stride_h = args->q_stride[2];
+  sp.k_stride_page = args->k_stride[0]; sp.k_stride_slot = args->k_stride[1]; sp.k_stride_h = args->k_stride[2];
+  sp.v_stride_page = args->v_stride[0]; sp.v_stride_slot = args->v_stride[1]; sp.v_stride_h = args->v_stride[2];
+  sp.batch = args->batch; sp.heads = args->heads; sp.kv_heads = args->kv_heads;
+  sp.group = args->heads / args->kv_heads;
+  sp.page_size = args->page_size; sp.num_pages = args->num_pages;
+  sp.chunk_tokens = g.chunk; sp.chunks_per_rank = g.chunks_per_rank; sp.num_slots = g.num_slots;
+  sp.max_split = args->max_split_per_seq;
+  sp.scale_log2 = args->softmax_scale * 1.4426950408889634f;
+
+  // one launch per row-tile class, widest rows first (they carry the longest KV runs)
+  for (int cls = 2; cls >= 0; --cls) {
+    if (g.class_wgs[cls] == 0) continue;
+    int nb = 0;
+    int64_t wg = 0;
+    for (int i = 0; i < args->num_buckets; ++i) {
+      const pat_fwd_bucket& b = args->buckets[i];
+      if ((row_tiles(b.mnw[0]) >> 1) != cls || b.num_boxes == 0) continue;
+      BucketDev& d = sp.bucket[nb++];
+      d.q_table = b.q_table; d.block_table = b.block_table; d.num_seqs = b.num_seqs;
+      d.rank = b.rank; d.kv = b.kv;
+      d.q_stride = (int32_t)b.q_table_stride; d.bt_stride = (int32_t)b.block_table_stride;
+      d.num_boxes = b.num_boxes; d.max_seqs = b.max_seqs; d.max_blocks = b.max_blocks;
+      d.chunks = g.bucket_chunks[i];
+      d.wg_begin = (int32_t)wg;
+      wg += (int64_t)b.num_boxes * d.chunks * args->kv_heads;
+    }
+    sp.num_buckets = nb;
+    sp.total_wgs = (int32_t)wg;
+    const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, 1 << cls, (unsigned)wg, stream, sp);
+    if (e != hipSuccess) return hip_fail(e, "split kernel launch");
+  }
+
+  MergeParams mp;
+  std::memset(&mp, 0, sizeof(mp));
+  mp.o_part = o_part; mp.lse_part = lse_part; mp.num_split_per_seq = args->num_split_per_seq;
+  mp.out = args->out; mp.lse_out = args->lse_out;
+  mp.o_stride_b = args->o_stride[0]; mp.o_stride_h = args->o_stride[2];
+  mp.batch = args->batch; mp.heads = args->heads; mp.head_dim = args->head_dim;
+  mp.chunks_per_rank = g.chunks_per_rank; mp.num_slots = g.num_slots; mp.max_split = args->max_split_per_seq;
+  const hipError_t e = launch_merge(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, mp);
+  if (e != hipSuccess) return hip_fail(e, "merge kernel launch");
+  return PAT_OK;
+}
+
+}  // extern "C"

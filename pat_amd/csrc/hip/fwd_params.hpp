@@ -1,0 +1,62 @@
+// Kernel-argument structures shared by the host launcher and the gfx950 kernels.
+#pragma once
+#include <cstdint>
+
+namespace pat {
+
+constexpr int kMaxBuckets = 12;    // the reference dispatches 12 tile shapes (static_switch.h:3-66)
+constexpr int kWaves = 4;          // waves per split-kernel workgroup
+constexpr int kThreads = kWaves * 64;
+constexpr int kStepTokens = 32;    // KV tokens one wave consumes per loop iteration
+constexpr int kMaxChunkPages = 128; // page ids one workgroup stages in LDS
+
+// One tile bucket as the split kernel sees it.
+struct BucketDev {
+  const int32_t* q_table;
+  const int32_t* block_table;
+  const int32_t* num_seqs;
+  const int32_t* rank;
+  const int32_t* kv;
+  int32_t q_stride;      // elements between q_table rows
+  int32_t bt_stride;     // elements between block_table rows
+  int32_t num_boxes;
+  int32_t max_seqs;      // valid q_table columns
+  int32_t max_blocks;    // valid block_table columns
+  int32_t chunks;        // workgroups along the KV axis reserved per box
+  int32_t wg_begin;      // first workgroup of this bucket inside its launch
+  int32_t pad_;
+};
+
+struct SplitParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  float* o_part;     // [batch, heads, num_slots, head_dim] fp32, normalised partial outputs
+  float* lse_part;   // [batch, heads, num_slots] fp32, natural-log LSE of each partial (-inf = empty)
+  int64_t q_stride_b, q_stride_h;              // elements
+  int64_t k_stride_page, k_stride_slot, k_stride_h;
+  int64_t v_stride_page, v_stride_slot, v_stride_h;
+  int32_t batch, heads, kv_heads, group;       // group = heads / kv_heads
+  int32_t page_size, num_pages;
+  int32_t chunk_tokens;     // KV tokens per workgroup (multiple of 32 and of page_size)
+  int32_t chunks_per_rank;  // slots reserved per CTA_rank
+  int32_t num_slots;        // max_split_per_seq * chunks_per_rank
+  int32_t max_split;
+  int32_t total_wgs;
+  float scale_log2;         // softmax_scale * log2(e)
+  int32_t num_buckets;
+  BucketDev bucket[kMaxBuckets];
+};
+
+struct MergeParams {
+  const float* o_part;
+  const float* lse_part;
+  const int32_t* num_split_per_seq;
+  void* out;
+  float* lse_out;           // may be null
+  int64_t o_stride_b, o_stride_h;
+  int32_t batch, heads, head_dim;
+  int32_t chunks_per_rank, num_slots, max_split;
+};
+
+}  // namespace pat

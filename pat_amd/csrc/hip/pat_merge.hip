@@ -1,0 +1,87 @@
+// Merge kernel for gfx950: combines the partial outputs of one (sequence, query head)
+// into the final attention row.
+//
+// Contract (the reference's gather_kernel, csrc/pat_fwd_kernel.h:314-467): with
+// partial results (O_i, LSE_i), LSE = M + ln(sum_i e^(LSE_i - M)), M = max_i LSE_i and
+// out = sum_i e^(LSE_i - LSE) * O_i, cast to the output type; the final LSE is natural
+// log of the scaled-logit sum.
+//
+// One wave64 per (sequence, head): lanes first scan the row's slot LSEs (slots that
+// no workgroup filled hold -inf and get weight 0), then each lane accumulates
+// head_dim/64 columns over the filled slots, so every partial row is read as one
+// contiguous 256- or 512-byte segment.
+#include <hip/hip_runtime.h>
+
+#include "fwd_params.hpp"
+
+namespace pat {
+
+template <typename T, int D>
+__global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
+  constexpr int CPL = D / 64;  // columns per lane
+  const int lane = threadIdx.x & 63;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= (int64_t)p.batch * p.heads) return;
+  const int s = (int)(pair / p.heads);
+  const int hq = (int)(pair % p.heads);
+
+  int nsplit = p.num_split_per_seq[s];
+  nsplit = nsplit < 0 ? 0 : (nsplit > p.max_split ? p.max_split : nsplit);
+  const int nslots = nsplit * p.chunks_per_rank;  // slots are rank-major
+  const float* __restrict__ lse = p.lse_part + pair * p.num_slots;
+  const float* __restrict__ op = p.o_part + pair * (int64_t)p.num_slots * D;
+
+  // pass 1: global max and sum of the slot LSEs
+  float mx = -__builtin_inff();
+  for (int i = lane; i < nslots; i += 64) mx = fmaxf(mx, lse[i]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  float sum = 0.f;
+  if (mx > -__builtin_inff())
+    for (int i = lane; i < nslots; i += 64) sum += __expf(lse[i] - mx);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  const float total = (sum > 0.f) ? mx + logf(sum) : -__builtin_inff();
+
+  // pass 2: weighted sum of the filled slots
+  float acc[CPL];
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
+  for (int base = 0; base < nslots; base += 64) {
+    const int i = base + lane;
+    const float mine = (i < nslots) ? lse[i] : -__builtin_inff();
+    const float w_mine = (mine > -__builtin_inff()) ? __expf(mine - total) : 0.f;
+    unsigned long long live = __ballot(w_mine > 0.f);
+    while (live) {
+      const int j = __builtin_ctzll(live);
+      live &= live - 1;
+      const float w = __shfl(w_mine, j);
+      const float* row = op + (int64_t)(base + j) * D + lane * CPL;
+      if (CPL == 2) {
+        const float2 v = *(const float2*)row;
+        acc[0] += w * v.x;
+        acc[CPL - 1] += w * v.y;
+      } else {
+        acc[0] += w * row[0];
+      }
+    }
+  }
+
+  T* dst = (T*)p.out + (int64_t)s * p.o_stride_b + (int64_t)hq * p.o_stride_h + lane * CPL;
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) dst[c] = (T)acc[c];
+  if (p.lse_out != nullptr && lane == 0) p.lse_out[pair] = total;
+}
+
+// Host launcher: one wave per (sequence, query head), four per workgroup.
+hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params) {
+  const int64_t pairs = (int64_t)params.batch * params.heads;
+  const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+  void (*fn)(const MergeParams);
+  if (bf16) fn = head_dim == 64 ? pat_merge_kernel<__bf16, 64> : pat_merge_kernel<__bf16, 128>;
+  else fn = head_dim == 64 ? pat_merge_kernel<_Float16, 64> : pat_merge_kernel<_Float16, 128>;
+  hipLaunchKernelGGL(fn, grid, block, 0, stream, params);
+  return hipGetLastError();
+}
+
+}  // namespace pat
