@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of prefix-aware decode attention on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+A step is one call of the hot path (pat_fwd_launch through the C ABI of libpat_amd: split
+kernel + merge kernel) on one decode batch of the named workload, with the plan already on
+the device. Synthetic, seeded N(0,1) inputs are resident in HBM before the timed region; the
+KV cache is rotated over several copies whose total size exceeds the 256 MB Infinity Cache so
+that consecutive steps cannot be served from it.
+
+Prints ONE JSON line. `value` is unique-KV bytes / time per call (GB/s); `ms_per_step` is the
+latency per call. `roofline` covers the split kernel (HBM-bound): algorithmic bytes = unique
+KV bytes of the batch, duration = mean split-kernel time from HIP events on the launch stream.
+`cpu_baseline` times this repository's CPU restatement of the reference's PyTorch attention
+on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+INFINITY_CACHE_BYTES = 256 << 20
+
+WORKLOAD_TEXT = {
+    "c1": "8 req, 256 shared + 32 private tokens, 8/8 heads, d64, fp16",
+    "c2": "Llama-3-8B shape: batch 64, 2048-token shared prefix + U[64,512] suffix, 32/8 heads, d128, bf16, page 16",
+    "c3": "batch 128, 1024 root + 8x512 mid + U[128,1024] leaves, 32/8 heads, d128, fp16",
+    "c4": "batch 256, forest of 16 roots, depth<=4, 16/16 heads, d64, fp16",
+    "c5a": "Llama-3-70B layer shape: batch 32, 16384 shared + U[256,2048], 64/8 heads, d128, bf16",
+    "c5b": "batch 32 independent 4096-token contexts, 64/8 heads, d128, bf16",
+}
+
+
+class Hip:
+    """hipEvent timing on a given stream, straight from the HIP runtime."""
+
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        self.lib.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.lib.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.lib.hipEventSynchronize.argtypes = [C.c_void_p]
+
+    def event(self) -> C.c_void_p:
+        e = C.c_void_p()
+        assert self.lib.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream) -> None:
+        assert self.lib.hipEventRecord(e, C.c_void_p(stream)) == 0
+
+    def ms(self, a, b) -> float:
+        out = C.c_float()
+        assert self.lib.hipEventSynchronize(b) == 0
+        assert self.lib.hipEventElapsedTime(C.byref(out), a, b) == 0
+        return out.value
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOAD_TEXT))
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-oblivious", action="store_true")
+    ap.add_argument("--kernel-loop-only", action="store_true",
+                    help="run only warmup + timed steps (for rocprofv3 runs)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no cross-GPU step); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from pat_amd import PrefixTreeCPP, _lib, _prefix_attn, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs an AMD GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+    hip = Hip()
+
+    w = workloads.make(a.workload, seed=a.seed)
+    cache_bytes = w.kv_bytes(w.num_blocks * w.page_size)
+    copies = max(2, min(16, math.ceil(2.5 * INFINITY_CACHE_BYTES / cache_bytes)))
+    q, ks, vs = w.tensors(dev, copies=copies)
+    scale = 1.0 / math.sqrt(w.head_dim)
+
+    t0 = time.perf_counter()
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    plan_ms = (time.perf_counter() - t0) * 1e3
+    info = tree.kernel_info
+    info.to_gpu(dev)
+
+    out = torch.empty_like(q)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def prepare(plan_kw, slots):
+        launches = []
+        for i in range(copies):
+            L = _prefix_attn._prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
+                                      plan_kw["block_tables"], plan_kw["num_seqs_per_CTAs"], plan_kw["CTA_ranks"],
+                                      plan_kw["kv_in_CTAs"], plan_kw["MNW"], plan_kw["max_split_per_seq"],
+                                      plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots)
+            launches.append(L)
+        ws = torch.empty(max(L.need for L in launches), dtype=torch.uint8, device=dev)
+        for L in launches:
+            L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), ws.numel()
+        return launches, ws
+
+    pat_kw = dict(num_split_per_seq=info.num_split_per_seq, query_tables=info.q_tables,
+                  block_tables=info.block_tables, num_seqs_per_CTAs=info.num_seqs_per_CTAs,
+                  CTA_ranks=info.CTA_ranks, kv_in_CTAs=info.kv_in_CTAs, MNW=info.MNWs,
+                  max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
+                  max_blocks_in_CTA=info.max_blocks_in_CTA)
+    pat_launches, pat_ws = prepare(pat_kw, info.slot_tables)
+
+    def step(launches, i):
+        rc = lib.pat_fwd_launch(C.byref(launches[i % copies].args), C.c_void_p(stream))
+        if rc != 0:
+            raise RuntimeError(_lib.last_error())
+
+    def timed(launches, steps, warmup):
+        for i in range(warmup):
+            step(launches, i)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for i in range(steps):
+            step(launches, warmup + i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) * 1e3 / steps
+
+    ms_per_step = timed(pat_launches, a.steps, a.warmup)
+    if a.kernel_loop_only:
+        print(json.dumps({"ms_per_step": ms_per_step, "steps": a.steps, "warmup": a.warmup}))
+        return
+
+    # per-kernel durations from HIP events on the launch stream (same step sequence)
+    n_ev = min(a.steps, 100)
+    ev = [(hip.event(), hip.event(), hip.event()) for _ in range(n_ev)]
+    for i, (e0, e1, e2) in enumerate(ev):
+        L = pat_launches[i % copies]
+        L.args.split_done_event = e1
+        hip.record(e0, stream)
+        step(pat_launches, i)
+        hip.record(e2, stream)
+        L.args.split_done_event = None
+    torch.cuda.synchronize()
+    split_ms = sorted(hip.ms(e0, e1) for e0, e1, _ in ev)
+    merge_ms = sorted(hip.ms(e1, e2) for _, e1, e2 in ev)
+    call_ms = sorted(hip.ms(e0, e2) for e0, _, e2 in ev)
+    mean = lambda xs: sum(xs) / len(xs)
+    median = lambda xs: xs[len(xs) // 2]
+
+    unique_bytes = w.unique_kv_bytes
+    value = unique_bytes / (ms_per_step * 1e-3) / 1e9
+    split_mean_ms = mean(split_ms)
+    achieved = unique_bytes / (split_mean_ms * 1e-3) / 1e9
+
+    geo = _lib.FwdGeometry()
+    lib.pat_fwd_geometry_of(C.byref(pat_launches[0].args), C.byref(geo))
+
+    result = {
+        "metric": "decode-attn us/call + unique-KV HBM GB/s (% of peak), Llama-3-8B shapes",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {WORKLOAD_TEXT[a.workload]}", "batch": w.batch,
+                   "heads": w.heads, "kv_heads": w.kv_heads, "head_dim": w.head_dim, "page_size": w.page_size,
+                   "seed": a.seed, "unique_kv_tokens": w.unique_tokens, "total_kv_tokens": w.total_tokens,
+                   "kv_cache_copies_rotated": copies},
+        "us_per_call": round(ms_per_step * 1e3, 3),
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "unique_kv_bytes": unique_bytes,
+        "oblivious_kv_bytes": w.kv_bytes(w.total_tokens),
+        "event_us": {"call_median": round(median(call_ms) * 1e3, 3), "split_mean": round(split_mean_ms * 1e3, 3),
+                     "split_median": round(median(split_ms) * 1e3, 3), "merge_mean": round(mean(merge_ms) * 1e3, 3)},
+        "geometry": {"chunk_tokens": geo.chunk_tokens, "tall_chunk_tokens": geo.tall_chunk_tokens,
+                     "chunks_per_rank": geo.chunks_per_rank, "workgroups": geo.num_workgroups},
+        "plan_build_ms_host": round(plan_ms, 3),
+        "roofline": {"bound": "hbm", "kernel": "pat_split_kernel", "achieved": round(achieved, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None},
+    }
+
+    # measured HBM traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE), if recorded
+    traffic_file = os.path.join(ROOT, "profiles", f"traffic_{a.workload}.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            result["roofline"]["traffic"] = json.load(f).get("bytes_per_launch")
+
+    if not a.no_oblivious:
+        ob = workloads.oblivious_plan(w, dev)
+        ob_kw = {k: ob[k] for k in pat_kw}
+        ob_launches, ob_ws = prepare(ob_kw, None)
+        ob_ms = timed(ob_launches, a.steps, a.warmup)
+        result["oblivious_us_per_call"] = round(ob_ms * 1e3, 3)
+        result["speedup_vs_oblivious"] = round(ob_ms / ms_per_step, 3)
+
+    if not a.no_cpu_baseline:
+        from oracle import attn_oracle
+        qc, kc, vc = q.cpu(), ks[0].cpu(), vs[0].cpu()
+        cores = os.cpu_count() or 1
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        torch.set_num_threads(cores)
+        attn_oracle.paged_attention_ref(qc, kc, vc, w.rows, w.seq_lens, scale)    # warm-up
+        runs, t_cpu = 0, 0.0
+        while runs < 5 and t_cpu < 20.0:
+            t = time.perf_counter()
+            attn_oracle.paged_attention_ref(qc, kc, vc, w.rows, w.seq_lens, scale)
+            t_cpu += time.perf_counter() - t
+            runs += 1
+        cpu_s = t_cpu / runs
+        result["cpu_baseline"] = {"value": round(unique_bytes / cpu_s / 1e9, 4), "unit": "GB/s",
+                                  "cores": torch.get_num_threads(), "kind": "port",
+                                  "us_per_call": round(cpu_s * 1e6, 1),
+                                  "sample": f"whole {a.workload} batch, fp32 PyTorch restatement of the reference's "
+                                            f"attention_ref over gathered dense KV, mean of {runs} runs after 1 warm-up"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -97,6 +97,12 @@ typedef struct pat_bucket_view {
   const int32_t* num_seqs;    /* [num_boxes]  num_seqs_per_CTA                */
   const int32_t* rank;        /* [num_boxes]  CTA_rank                        */
   const int32_t* kv;          /* [num_boxes]  kv_in_CTA (tokens)              */
+  /* Not part of the reference plan: for box b and its j-th sequence s, the number of
+   * earlier boxes of the plan (bucket order, then box order) that contain s. Unlike
+   * CTA_rank it is unique per (sequence, box) by construction, also on forests where
+   * the reference hands one rank to two boxes of a sequence. Same shape/padding as
+   * q_table. */
+  const int32_t* q_slot;      /* [num_boxes, max_seqs]                        */
 } pat_bucket_view;
 
 typedef struct pat_plan_view {
@@ -158,6 +164,8 @@ typedef struct pat_fwd_bucket {
   const int32_t* num_seqs;    /* [num_boxes]                                  */
   const int32_t* rank;        /* [num_boxes]                                  */
   const int32_t* kv;          /* [num_boxes]                                  */
+  const int32_t* q_slot;      /* optional [num_boxes, q_table_stride] (see     */
+                              /* pat_bucket_view.q_slot); NULL: use CTA_rank   */
   int64_t q_table_stride;     /* elements between rows                        */
   int64_t block_table_stride; /* elements between rows                        */
   int32_t num_boxes;
@@ -196,6 +204,8 @@ typedef struct pat_fwd_args {
   const pat_fwd_bucket* buckets; /* host array [num_buckets]                  */
   void* workspace;               /* device scratch, 256-byte aligned          */
   size_t workspace_bytes;
+  void* split_done_event;        /* optional hipEvent_t recorded on the stream between the   */
+                                 /* split kernel and the merge kernel (timing aid), or NULL  */
 } pat_fwd_args;
 
 /* Argument checks of csrc/api.h:129-181 that need no GPU (dtype enum, head_dim,
@@ -216,11 +226,11 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
 
 /* Description of the launch geometry chosen for `args` (for benchmarks/tests). */
 typedef struct pat_fwd_geometry {
-  int32_t chunk_tokens;     /* KV tokens one workgroup streams                */
-  int32_t chunks_per_rank;  /* partial slots reserved per CTA_rank            */
-  int32_t num_slots;        /* max_split_per_seq * chunks_per_rank            */
-  int32_t num_launches;     /* split-kernel launches (one per row-tile class) */
-  int64_t num_workgroups;   /* total split-kernel workgroups                  */
+  int32_t chunk_tokens;      /* KV tokens one workgroup streams (boxes <= 16 rows) */
+  int32_t tall_chunk_tokens; /* same for boxes of 17..64 rows                      */
+  int32_t chunks_per_rank;   /* partial slots reserved per box                     */
+  int32_t num_slots;         /* max_split_per_seq * chunks_per_rank                */
+  int64_t num_workgroups;    /* split-kernel workgroups                            */
 } pat_fwd_geometry;
 int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out);
 

@@ -42,7 +42,7 @@ class BucketView(C.Structure):
     _fields_ = [("mnw", C.c_int32 * 3), ("num_boxes", C.c_int32), ("max_seqs", C.c_int32),
                 ("max_blocks", C.c_int32), ("q_table", i32p), ("block_table", i32p),
                 ("q_len", i32p), ("block_len", i32p), ("num_seqs", i32p), ("rank", i32p),
-                ("kv", i32p)]
+                ("kv", i32p), ("q_slot", i32p)]
 
 
 class PlanView(C.Structure):
@@ -54,7 +54,7 @@ class PlanView(C.Structure):
 
 class FwdBucket(C.Structure):
     _fields_ = [("q_table", C.c_void_p), ("block_table", C.c_void_p), ("num_seqs", C.c_void_p),
-                ("rank", C.c_void_p), ("kv", C.c_void_p),
+                ("rank", C.c_void_p), ("kv", C.c_void_p), ("q_slot", C.c_void_p),
                 ("q_table_stride", C.c_int64), ("block_table_stride", C.c_int64),
                 ("num_boxes", C.c_int32), ("max_seqs", C.c_int32), ("max_blocks", C.c_int32),
                 ("mnw", C.c_int32 * 3)]
@@ -72,12 +72,13 @@ class FwdArgs(C.Structure):
                 ("max_split_per_seq", C.c_int32), ("max_seqs_in_box", C.c_int32),
                 ("max_blocks_in_box", C.c_int32), ("softmax_scale", C.c_float),
                 ("num_buckets", C.c_int32), ("buckets", C.POINTER(FwdBucket)),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+                ("split_done_event", C.c_void_p)]
 
 
 class FwdGeometry(C.Structure):
-    _fields_ = [("chunk_tokens", C.c_int32), ("chunks_per_rank", C.c_int32),
-                ("num_slots", C.c_int32), ("num_launches", C.c_int32),
+    _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
+                ("chunks_per_rank", C.c_int32), ("num_slots", C.c_int32),
                 ("num_workgroups", C.c_int64)]
 
 

@@ -39,6 +39,9 @@ class KernelInfo:
         self.num_seqs_per_CTAs: List[torch.Tensor] = []
         self.CTA_ranks: List[torch.Tensor] = []
         self.kv_in_CTAs: List[torch.Tensor] = []
+        # not in the reference: per (box, sequence) the box's ordinal among that sequence's
+        # boxes; the kernels use it as a collision-free partial-result slot
+        self.slot_tables: List[torch.Tensor] = []
         self.MNWs: List[List[int]] = []
         self.num_split_per_seq: torch.Tensor = torch.empty(0, dtype=torch.int32)
         self.max_split_per_seq = 0
@@ -58,6 +61,7 @@ class KernelInfo:
         self.num_seqs_per_CTAs = [move(t) for t in self.num_seqs_per_CTAs]
         self.CTA_ranks = [move(t) for t in self.CTA_ranks]
         self.kv_in_CTAs = [move(t) for t in self.kv_in_CTAs]
+        self.slot_tables = [move(t) for t in self.slot_tables]
         self.num_split_per_seq = move(self.num_split_per_seq)
         self._launch_cache.clear()
 
@@ -81,6 +85,7 @@ class KernelInfo:
             ki.num_seqs_per_CTAs.append(vec(bk.num_seqs))
             ki.CTA_ranks.append(vec(bk.rank))
             ki.kv_in_CTAs.append(vec(bk.kv))
+            ki.slot_tables.append(mat(bk.q_slot, ws))
         ki.num_split_per_seq = torch.from_numpy(
             np.ctypeslib.as_array(view.num_split_per_seq, shape=(view.batch,)).copy())
         ki.max_split_per_seq = view.max_split_per_seq
@@ -142,7 +147,7 @@ class _Launch:
 
 
 def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MNW, max_split,
-             max_seqs, max_blocks, scale, out, lse) -> _Launch:
+             max_seqs, max_blocks, scale, out, lse, slot_tables=None) -> _Launch:
     lib = _lib.load()
     # --- checks that need tensor metadata (csrc/api.h:131-181, :256-277) -----------------
     _check(q.dtype in (torch.float16, torch.bfloat16), "only support fp16 and bf16 data type")
@@ -165,6 +170,9 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
     nb = len(MNW)
     _check(all(len(x) == nb for x in (q_tables, block_tables, num_seqs, ranks, kvs)),
            "MNW and the per-bucket plan lists must have the same length")
+    if slot_tables is not None and len(slot_tables) == 0:
+        slot_tables = None
+    _check(slot_tables is None or len(slot_tables) == nb, "slot_tables must have one entry per bucket")
 
     L = _Launch()
     L.buckets = (_lib.FwdBucket * max(nb, 1))()
@@ -182,6 +190,11 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
         fb = L.buckets[i]
         fb.q_table, fb.block_table = qt.data_ptr(), bt.data_ptr()
         fb.num_seqs, fb.rank, fb.kv = ns.data_ptr(), rk.data_ptr(), kv.data_ptr()
+        if slot_tables is not None:
+            st = slot_tables[i]
+            _check(st.is_cuda and st.dtype == torch.int32 and tuple(st.shape) == tuple(qt.shape)
+                   and st.stride() == qt.stride(), "slot_tables must match query_tables (CUDA int32, same layout)")
+            fb.q_slot = st.data_ptr()
         fb.q_table_stride = qt.stride(0) if ctas > 1 else max(qt.shape[1], 1)
         fb.block_table_stride = bt.stride(0) if ctas > 1 else max(bt.shape[1], 1)
         fb.num_boxes, fb.max_seqs, fb.max_blocks = ctas, qt.shape[1], bt.shape[1]
@@ -207,7 +220,8 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
     L.args, L.need = a, need.value
     # plan tensors stay referenced as long as the prepared launch does; q/k/v/out are the
     # caller's for the duration of the call only
-    L.keep = (num_split, list(q_tables), list(block_tables), list(num_seqs), list(ranks), list(kvs))
+    L.keep = (num_split, list(q_tables), list(block_tables), list(num_seqs), list(ranks), list(kvs),
+              None if slot_tables is None else list(slot_tables))
     L.workspace = None
     return L
 
@@ -231,9 +245,13 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                   max_blocks_in_CTA, softmax_scale, out, timing_=None)
     Tree form:   (q, k_cache_paged, v_cache_paged, tree, softmax_scale, out)
     Both accept the extra keyword `softmax_lse` (float32 [batch, heads]) to receive the
-    natural-log LSE, which the reference computes but does not return.
+    natural-log LSE, which the reference computes but does not return. The table form also
+    accepts `slot_tables` (`KernelInfo.slot_tables`): with it, partial results are filed by each
+    box's ordinal within its sequence instead of by CTA_rank, which stays correct on batches
+    where the reference scheduler hands the same rank to two boxes of one sequence.
     """
     lse = kw.pop("softmax_lse", None)
+    slots = kw.pop("slot_tables", None)
     tree_names = ("tree", "softmax_scale", "out")
     table_names = ("num_split_per_seq", "query_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks",
                    "kv_in_CTAs", "MNW", "max_split_per_seq", "max_seqs_in_CTA", "max_blocks_in_CTA",
@@ -252,6 +270,8 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
         raise TypeError(f"prefix_attn_with_kvcache(): missing arguments {missing}")
 
     out = vals["out"]
+    for name, t in (("q", q), ("kcache", k_cache_paged), ("vcache", v_cache_paged)):
+        _check(isinstance(t, torch.Tensor) and t.is_cuda, f"{name} must be on CUDA")
     with torch.cuda.device(q.device):
         if is_tree:
             tree = vals["tree"]
@@ -265,7 +285,7 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                 L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, info.q_tables,
                              info.block_tables, info.num_seqs_per_CTAs, info.CTA_ranks, info.kv_in_CTAs,
                              info.MNWs, info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
-                             vals["softmax_scale"], out, lse)
+                             vals["softmax_scale"], out, lse, info.slot_tables)
                 if len(info._launch_cache) >= 256:
                     info._launch_cache.clear()
                 info._launch_cache[key] = L
@@ -273,5 +293,5 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
             L = _prepare(q, k_cache_paged, v_cache_paged, vals["num_split_per_seq"], vals["query_tables"],
                          vals["block_tables"], vals["num_seqs_per_CTAs"], vals["CTA_ranks"], vals["kv_in_CTAs"],
                          vals["MNW"], vals["max_split_per_seq"], vals["max_seqs_in_CTA"],
-                         vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse)
+                         vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse, slots)
         _run(L, q.device)

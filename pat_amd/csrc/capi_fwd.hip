@@ -15,7 +15,7 @@
 namespace pat {
 
 // defined next to the kernels (hip/pat_split.hip, hip/pat_merge.hip)
-hipError_t launch_split(bool bf16, int head_dim, int row_tiles, unsigned workgroups, hipStream_t stream,
+hipError_t launch_split(bool bf16, int head_dim, unsigned workgroups, hipStream_t stream,
                         const SplitParams& params);
 hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params);
 
@@ -34,13 +34,13 @@ inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = 
 inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 2 : 4); }
 
 struct Geometry {
-  int chunk = 0;             // tokens per workgroup
+  int chunk = 0;             // tokens per workgroup, boxes of <= 16 rows
+  int tall_chunk = 0;        // tokens per workgroup, boxes of 17..64 rows
   int chunks_per_rank = 0;   // widest bucket's chunk count
   int num_slots = 0;
+  int bucket_chunk[kMaxBuckets] = {0};
   int bucket_chunks[kMaxBuckets] = {0};
-  int64_t class_wgs[3] = {0, 0, 0};  // workgroups per row-tile class (1, 2, 4 tiles)
   int64_t total_wgs = 0;
-  int launches = 0;
 };
 
 int check_args(const pat_fwd_args* a) {
@@ -104,50 +104,46 @@ int check_args(const pat_fwd_args* a) {
   return PAT_OK;
 }
 
-// Launch geometry: one chunk size for the whole call. Sized so the device sees a few
-// workgroups per CU; a bucket reserves ceil(widest box / chunk) workgroups per box.
+// Launch geometry. A workgroup streams one chunk of one box for one kv head; a bucket reserves
+// ceil(widest box / chunk) workgroups per box (those past a box's real length exit at once).
+//  * boxes of <= 16 rows split the chunk's 32-token steps over the 4 waves: the chunk is sized
+//    so that the device sees a few workgroups per CU, between 128 and 1024 tokens;
+//  * boxes of 17..64 rows give every wave the whole chunk (rows are split instead) and write
+//    16 KB..32 KB of partial output per workgroup, so they use a fixed, longer chunk.
+// PAT_CHUNK_TOKENS / PAT_TALL_CHUNK_TOKENS override both (tuning aid).
 int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   const int page = a->page_size;
   const int64_t unit = (int64_t)page * kStepTokens / gcd64(page, kStepTokens);  // lcm(page, 32)
-  int64_t total = 0, widest = 0;
-  for (int i = 0; i < a->num_buckets; ++i) {
-    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-    total += tok * a->buckets[i].num_boxes * a->kv_heads;
-    widest = std::max(widest, tok);
-  }
-  int64_t chunk = 0;
+  auto round_unit = [&](int64_t c) { return std::max<int64_t>(unit, ceil_div64(c, unit) * unit); };
+  int64_t short_total = 0;
+  for (int i = 0; i < a->num_buckets; ++i)
+    if (row_tiles(a->buckets[i].mnw[0]) == 1)
+      short_total += (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
+  int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
-  if (chunk <= 0) {
-    // aim at ~4 workgroups per CU, between 128 and 1024 tokens each
-    chunk = total / (4 * kNumCUs);
-    chunk = std::max<int64_t>(128, std::min<int64_t>(1024, chunk));
-  }
-  chunk = std::max<int64_t>(unit, ceil_div64(chunk, unit) * unit);
-  // bounded slot count per rank, and page ids of a chunk must fit their LDS table
-  while (ceil_div64(widest, chunk) > kMaxChunksPerRank) chunk += unit;
-  if (chunk / page > kMaxChunkPages) {
-    chunk = (int64_t)kMaxChunkPages * page / unit * unit;
-    if (chunk <= 0 || ceil_div64(widest, chunk) > kMaxChunksPerRank)
-      return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
-  }
-  g->chunk = (int)chunk;
+  if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
+  if (chunk <= 0) chunk = std::max<int64_t>(128, std::min<int64_t>(1024, short_total / (4 * kNumCUs)));
+  if (tall <= 0) tall = 256;
+  const int64_t cap = (int64_t)kMaxChunkPages * page / unit * unit;  // page ids of a chunk sit in LDS
+  if (cap <= 0) return fail(PAT_ERR_INVALID, "page size too large for one workgroup");
   g->chunks_per_rank = 1;
-  for (int i = 0; i < a->num_buckets; ++i) {
-    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-    const int c = (int)std::max<int64_t>(1, ceil_div64(tok, chunk));
-    g->bucket_chunks[i] = c;
-    g->chunks_per_rank = std::max(g->chunks_per_rank, c);
-    const int cls = row_tiles(a->buckets[i].mnw[0]) >> 1;  // 1,2,4 -> 0,1,2
-    g->class_wgs[cls] += (int64_t)a->buckets[i].num_boxes * c * a->kv_heads;
-  }
-  g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
   g->total_wgs = 0;
-  g->launches = 0;
-  for (int c = 0; c < 3; ++c) {
-    if (g->class_wgs[c] > INT32_MAX) return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
-    g->total_wgs += g->class_wgs[c];
-    g->launches += g->class_wgs[c] > 0;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const bool is_tall = row_tiles(a->buckets[i].mnw[0]) > 1;
+    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+    int64_t c = round_unit(is_tall ? tall : chunk);
+    while (ceil_div64(tok, c) > kMaxChunksPerRank) c += unit;   // bounded slots per box
+    if (c > cap) return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
+    const int n = (int)std::max<int64_t>(1, ceil_div64(tok, c));
+    g->bucket_chunk[i] = (int)c;
+    g->bucket_chunks[i] = n;
+    g->chunks_per_rank = std::max(g->chunks_per_rank, n);
+    g->total_wgs += (int64_t)a->buckets[i].num_boxes * n * a->kv_heads;
   }
+  g->chunk = (int)round_unit(chunk);
+  g->tall_chunk = (int)round_unit(tall);
+  g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
+  if (g->total_wgs > INT32_MAX) return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   return PAT_OK;
 }
 
@@ -175,9 +171,9 @@ int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out) {
   pat::Geometry g;
   if (int rc = pat::plan_geometry(args, &g)) return rc;
   out->chunk_tokens = g.chunk;
+  out->tall_chunk_tokens = g.tall_chunk;
   out->chunks_per_rank = g.chunks_per_rank;
   out->num_slots = g.num_slots;
-  out->num_launches = g.launches;
   out->num_workgroups = g.total_wgs;
   return PAT_OK;
 }
@@ -219,31 +215,39 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   sp.batch = args->batch; sp.heads = args->heads; sp.kv_heads = args->kv_heads;
   sp.group = args->heads / args->kv_heads;
   sp.page_size = args->page_size; sp.num_pages = args->num_pages;
-  sp.chunk_tokens = g.chunk; sp.chunks_per_rank = g.chunks_per_rank; sp.num_slots = g.num_slots;
+  sp.chunks_per_rank = g.chunks_per_rank; sp.num_slots = g.num_slots;
   sp.max_split = args->max_split_per_seq;
   sp.scale_log2 = args->softmax_scale * 1.4426950408889634f;
 
-  // one launch per row-tile class, widest rows first (they carry the longest KV runs)
-  for (int cls = 2; cls >= 0; --cls) {
-    if (g.class_wgs[cls] == 0) continue;
+  // one launch over all buckets, in plan order (tall, long boxes come first in the default order)
+  {
     int nb = 0;
     int64_t wg = 0;
     for (int i = 0; i < args->num_buckets; ++i) {
       const pat_fwd_bucket& b = args->buckets[i];
-      if ((row_tiles(b.mnw[0]) >> 1) != cls || b.num_boxes == 0) continue;
+      if (b.num_boxes == 0) continue;
       BucketDev& d = sp.bucket[nb++];
       d.q_table = b.q_table; d.block_table = b.block_table; d.num_seqs = b.num_seqs;
-      d.rank = b.rank; d.kv = b.kv;
+      d.rank = b.rank; d.kv = b.kv; d.q_slot = b.q_slot;
       d.q_stride = (int32_t)b.q_table_stride; d.bt_stride = (int32_t)b.block_table_stride;
       d.num_boxes = b.num_boxes; d.max_seqs = b.max_seqs; d.max_blocks = b.max_blocks;
+      d.chunk_tokens = g.bucket_chunk[i];
       d.chunks = g.bucket_chunks[i];
+      d.row_tiles = row_tiles(b.mnw[0]);
       d.wg_begin = (int32_t)wg;
       wg += (int64_t)b.num_boxes * d.chunks * args->kv_heads;
     }
     sp.num_buckets = nb;
     sp.total_wgs = (int32_t)wg;
-    const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, 1 << cls, (unsigned)wg, stream, sp);
-    if (e != hipSuccess) return hip_fail(e, "split kernel launch");
+    if (wg > 0) {
+      const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, (unsigned)wg, stream, sp);
+      if (e != hipSuccess) return hip_fail(e, "split kernel launch");
+    }
+  }
+
+  if (args->split_done_event != nullptr) {
+    const hipError_t e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), stream);
+    if (e != hipSuccess) return hip_fail(e, "hipEventRecord(split_done_event)");
   }
 
   MergeParams mp;

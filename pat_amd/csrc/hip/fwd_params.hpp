@@ -17,13 +17,16 @@ struct BucketDev {
   const int32_t* num_seqs;
   const int32_t* rank;
   const int32_t* kv;
-  int32_t q_stride;      // elements between q_table rows
+  const int32_t* q_slot; // optional [num_boxes, q_stride]: ordinal of the box among its sequence's boxes
+  int32_t q_stride;      // elements between q_table (and q_slot) rows
   int32_t bt_stride;     // elements between block_table rows
   int32_t num_boxes;
   int32_t max_seqs;      // valid q_table columns
   int32_t max_blocks;    // valid block_table columns
+  int32_t chunk_tokens;  // KV tokens per workgroup (multiple of 32 and of page_size)
   int32_t chunks;        // workgroups along the KV axis reserved per box
-  int32_t wg_begin;      // first workgroup of this bucket inside its launch
+  int32_t wg_begin;      // first workgroup of this bucket
+  int32_t row_tiles;     // 1: boxes of <= 16 rows (KV steps split over waves); >1: rows split over waves
   int32_t pad_;
 };
 
@@ -38,7 +41,6 @@ struct SplitParams {
   int64_t v_stride_page, v_stride_slot, v_stride_h;
   int32_t batch, heads, kv_heads, group;       // group = heads / kv_heads
   int32_t page_size, num_pages;
-  int32_t chunk_tokens;     // KV tokens per workgroup (multiple of 32 and of page_size)
   int32_t chunks_per_rank;  // slots reserved per CTA_rank
   int32_t num_slots;        // max_split_per_seq * chunks_per_rank
   int32_t max_split;

@@ -8,9 +8,13 @@
 // those tokens plus LSE = max + ln(sum) (csrc/softmax.h:169-188).
 //
 // Mapping to the hardware (this kernel's own design):
-//  * a workgroup = 4 wave64; each wave owns every 4th 32-token step of the chunk and
-//    runs an independent online softmax; the 4 partial states are combined through
-//    LDS at the end, so one (box, head, chunk) yields one partial row set.
+//  * a workgroup = 4 wave64 working on one (box, kv-head, chunk) in one of two ways:
+//      - boxes of up to 16 rows: each wave owns every 4th 32-token step of the chunk and
+//        runs an independent online softmax; the 4 states are combined through LDS;
+//      - boxes of 17..64 rows: wave w owns rows 16w..16w+15 over the whole chunk (the
+//        waves re-read the same K/V lines through L1), no combine needed.
+//    Either way one (box, head, chunk) yields one partial row set, every wave carries a
+//    single 16-row tile of state, and one launch covers all buckets.
 //  * S^T = K.Q^T on v_mfma_f32_16x16x32: K rows are the MFMA A operand, so a lane
 //    loads 16 contiguous bytes of one token straight from HBM into operand layout
 //    (no LDS for K). The accumulator layout of S^T is the B-operand layout of
@@ -51,7 +55,7 @@ template <> struct Elem<__bf16> {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 
-template <typename T, int D, int MT>
+template <typename T, int D>
 __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -91,17 +95,24 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
 
   const int G = p.group;
   const int rank = bk.rank[box];
-  if ((unsigned)rank >= (unsigned)p.max_split) return;  // malformed plan: touch nothing
   int nseq = bk.num_seqs[box];
   nseq = nseq < 0 ? 0 : (nseq > bk.max_seqs ? bk.max_seqs : nseq);
   int R = nseq * G;
-  if (R > MT * 16) R = MT * 16;
+  if (R > 64) R = 64;
+  const bool tall = bk.row_tiles > 1;            // rows split across waves instead of KV steps
+  const int row0 = tall ? wave * 16 : 0;         // first row of this wave's tile
   int kv = bk.kv[box];
   const int kv_cap = bk.max_blocks * p.page_size;
   kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
-  const int t_begin = chunk * p.chunk_tokens;
+  const int t_begin = chunk * bk.chunk_tokens;
   const int* __restrict__ qt = bk.q_table + (int64_t)box * bk.q_stride;
-  const int slot = rank * p.chunks_per_rank + chunk;
+  // Partial-slot ordinal of this box per sequence: the plan's own rank, or - when the caller
+  // supplies it - the box's ordinal among the boxes of that sequence (always collision-free).
+  const int* __restrict__ qs = bk.q_slot ? bk.q_slot + (int64_t)box * bk.q_stride : nullptr;
+  auto slot_base = [&](int j) -> int {
+    const int ord = qs ? qs[j] : rank;
+    return ((unsigned)ord < (unsigned)p.max_split) ? ord * p.chunks_per_rank : -1;
+  };
 
   // ---- slots of this rank nobody will fill are marked empty (-inf) -------------
   {
@@ -112,14 +123,15 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
     for (int idx = tid; idx < R * nmark; idx += kThreads) {
       const int r = idx / nmark, c = first + idx % nmark;
       const int s = qt[r / G];
-      if ((unsigned)s < (unsigned)p.batch) {
+      const int sb = slot_base(r / G);
+      if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
         const int hq = head * G + r % G;
-        p.lse_part[((int64_t)s * p.heads + hq) * p.num_slots + rank * p.chunks_per_rank + c] = neg_inf();
+        p.lse_part[((int64_t)s * p.heads + hq) * p.num_slots + sb + c] = neg_inf();
       }
     }
     if (empty) return;
   }
-  const int t_end = (kv < t_begin + p.chunk_tokens) ? kv : t_begin + p.chunk_tokens;
+  const int t_end = (kv < t_begin + bk.chunk_tokens) ? kv : t_begin + bk.chunk_tokens;
 
   // ---- page ids of the chunk -> LDS ---------------------------------------------
   const int page = p.page_size;
@@ -134,11 +146,10 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
     }
   }
 
-  // ---- Q rows as MFMA B operand (lane (g, n): row n, dims kk*32 + g*8 .. +7) -----
-  vec8 qreg[MT][KK];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int r = mt * 16 + n;
+  // ---- Q rows as MFMA B operand (lane (g, n): row row0 + n, dims kk*32 + g*8 .. +7) ----
+  vec8 qreg[KK];
+  {
+    const int r = row0 + n;
     int s = -1;
     if (r < R) s = qt[r / G];
     const bool ok = (unsigned)s < (unsigned)p.batch;
@@ -147,12 +158,16 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
     for (int kk = 0; kk < KK; ++kk) {
       u32x4 raw = u32x4{0u, 0u, 0u, 0u};
       if (ok) raw = *(const u32x4*)(qrow + kk * 32 + g * 8);
-      qreg[mt][kk] = __builtin_bit_cast(vec8, raw);
+      qreg[kk] = __builtin_bit_cast(vec8, raw);
     }
   }
   __syncthreads();  // s_pages visible
 
   const int nsteps = (t_end - t_begin + kStepTokens - 1) / kStepTokens;
+  // KV steps of this wave: every 4th one (short boxes) or all of them (tall boxes, where a
+  // wave whose rows are all padding has nothing to do)
+  const int st_first = tall ? ((row0 < R) ? 0 : nsteps) : wave;
+  const int st_stride = tall ? 1 : kWaves;
   const bool pow2 = (page & (page - 1)) == 0;
   const int pshift = 31 - __builtin_clz(page);
   const T* __restrict__ kbase = (const T*)p.k + (int64_t)head * p.k_stride_h;
@@ -188,20 +203,15 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
     }
   };
 
-  float m_run[MT], l_run[MT];
-  f32x4 acc_o[MT][DB];
+  float m_run = neg_inf(), l_run = 0.f;
+  f32x4 acc_o[DB];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    m_run[mt] = neg_inf();
-    l_run[mt] = 0.f;
-#pragma unroll
-    for (int db = 0; db < DB; ++db) acc_o[mt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int db = 0; db < DB; ++db) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   char* vstage = smem + wave * VSTAGE;
-  if (wave < nsteps) load_step(wave);
+  if (st_first < nsteps) load_step(st_first);
 
-  for (int st = wave; st < nsteps; st += kWaves) {
+  for (int st = st_first; st < nsteps; st += st_stride) {
     // current tile -> registers of this iteration; start fetching the next one
     u32x4 kcur[2][KK], vcur[NV];
 #pragma unroll
@@ -210,7 +220,7 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
       for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = kraw[a][kk];
 #pragma unroll
     for (int j = 0; j < NV; ++j) vcur[j] = vraw[j];
-    if (st + kWaves < nsteps) load_step(st + kWaves);
+    if (st + st_stride < nsteps) load_step(st + st_stride);
 
     // V tile -> this wave's LDS region, row-major with padded rows
 #pragma unroll
@@ -219,9 +229,47 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
       *(PAT_LDS u32x4*)((PAT_LDS char*)vstage + (piece / CPR) * RS + (piece % CPR) * 16) = vcur[j];
     }
 
-    // V^T operand: lane (g, n) of d-block db gets 8 tokens of column db*16 + n:
+    // S^T = K.Q^T for the two 16-token halves of the step
+    f32x4 sc[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        acc = E::mfma(__builtin_bit_cast(vec8, kcur[a][kk]), qreg[kk], acc);
+      sc[a] = acc * p.scale_log2;
+    }
+    const int t0 = t_begin + st * kStepTokens;
+    if (t0 + kStepTokens > t_end) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (t0 + a * 16 + g * 4 + i >= t_end) sc[a][i] = neg_inf();
+    }
+
+    // online softmax; the row's running max is shared by its 4 lanes, the sum stays per lane
+    float mx = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
+                     fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.f;
+    vec8 pv;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e = fast_exp2(sc[a][i] - m_new);
+        psum += e;
+        pv[a * 4 + i] = (T)e;
+      }
+    l_run = l_run * alpha + psum;
+
+    // O^T += V^T.P^T. V^T operand: lane (g, n) of d-block db gets 8 tokens of column db*16 + n:
     // tokens g*4..g*4+3 of each 16-token half, matching the accumulator layout of S^T.
-    vec8 vt[DB];
     {
       const int rrow = g * 4 + (n >> 2);
       const PAT_LDS char* src = (const PAT_LDS char*)vstage + rrow * RS + (n & 3) * 8;
@@ -230,122 +278,83 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + db * 32));
         s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + 16 * RS + db * 32));
         s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        vt[db] = __builtin_bit_cast(vec8, both);
-      }
-    }
-
-    const int t0 = t_begin + st * kStepTokens;
-    const bool tail = t0 + kStepTokens > t_end;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      f32x4 sc[2];
-#pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk)
-          acc = E::mfma(__builtin_bit_cast(vec8, kcur[a][kk]), qreg[mt][kk], acc);
-        sc[a] = acc * p.scale_log2;
-      }
-      if (tail) {
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (t0 + a * 16 + g * 4 + i >= t_end) sc[a][i] = neg_inf();
-      }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
-                       fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run[mt], mx);
-      const float alpha = fast_exp2(m_run[mt] - m_new);
-      m_run[mt] = m_new;
-      float psum = 0.f;
-      vec8 pv;
-#pragma unroll
-      for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = fast_exp2(sc[a][i] - m_new);
-          psum += e;
-          pv[a * 4 + i] = (T)e;
-        }
-      l_run[mt] = l_run[mt] * alpha + psum;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        acc_o[mt][db] = acc_o[mt][db] * alpha;
-        acc_o[mt][db] = E::mfma(vt[db], pv, acc_o[mt][db]);
+        acc_o[db] = acc_o[db] * alpha;
+        acc_o[db] = E::mfma(__builtin_bit_cast(vec8, both), pv, acc_o[db]);
       }
     }
   }
 
-  // ---- combine the 4 waves' states and write the partial -------------------------
-  float* cbuf = (float*)smem;
-  const int crow = tid >> 4;                 // row of the M-tile this thread finalises
-  const int ccol = (tid & 15) * (D / 16);    // its first column
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    float l = l_run[mt];
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
-    __syncthreads();  // staging / previous tile's combine buffer no longer read
-    if (g == 0) { s_m[wave][n] = m_run[mt]; s_l[wave][n] = l; }
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-      *(f32x4*)(cbuf + (wave * 16 + n) * OROW + db * 16 + g * 4) = acc_o[mt][db];
-    __syncthreads();
+  // the row's sum over all of this wave's tokens
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
 
-    const int r = mt * 16 + crow;
+  if (tall) {
+    // ---- tall box: this wave holds the finished rows row0..row0+15 of the chunk -----------
+    const int r = row0 + n;
     if (r < R) {
-      float mw[kWaves], mmax = neg_inf();
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) { mw[w] = s_m[w][crow]; mmax = fmaxf(mmax, mw[w]); }
-      float wsum = 0.f, wgt[kWaves];
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        wgt[w] = fast_exp2(mw[w] - mmax);   // a wave without steps has m = -inf -> weight 0
-        wsum += wgt[w] * s_l[w][crow];
-      }
-      const float inv = 1.f / wsum;
       const int s = qt[r / G];
-      if ((unsigned)s < (unsigned)p.batch) {
+      const int sb = slot_base(r / G);
+      if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
         const int hq = head * G + r % G;
-        const int64_t prow = ((int64_t)s * p.heads + hq) * p.num_slots + slot;
-        float* dst = p.o_part + prow * D + ccol;
+        const int64_t prow = ((int64_t)s * p.heads + hq) * p.num_slots + sb + chunk;
+        const float inv = 1.f / l_run;
+        float* dst = p.o_part + prow * D + g * 4;
 #pragma unroll
-        for (int c = 0; c < D / 16; c += 4) {
-          f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int w = 0; w < kWaves; ++w)
-            o += *(const f32x4*)(cbuf + (w * 16 + crow) * OROW + ccol + c) * wgt[w];
-          *(f32x4*)(dst + c) = o * inv;
-        }
-        if ((tid & 15) == 0)
-          p.lse_part[prow] = (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f;
+        for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
+        if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
       }
+    }
+    return;
+  }
+
+  // ---- short box: combine the 4 waves' states through LDS and write the partial -------------
+  float* cbuf = (float*)smem;
+  const int crow = tid >> 4;                 // row this thread finalises
+  const int ccol = (tid & 15) * (D / 16);    // its first column
+  __syncthreads();  // every wave is done with its V staging region
+  if (g == 0) { s_m[wave][n] = m_run; s_l[wave][n] = l_run; }
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+    *(f32x4*)(cbuf + (wave * 16 + n) * OROW + db * 16 + g * 4) = acc_o[db];
+  __syncthreads();
+
+  if (crow < R) {
+    float mw[kWaves], mmax = neg_inf();
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) { mw[w] = s_m[w][crow]; mmax = fmaxf(mmax, mw[w]); }
+    float wsum = 0.f, wgt[kWaves];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      wgt[w] = fast_exp2(mw[w] - mmax);   // a wave without steps has m = -inf -> weight 0
+      wsum += wgt[w] * s_l[w][crow];
+    }
+    const float inv = 1.f / wsum;
+    const int s = qt[crow / G];
+    const int sb = slot_base(crow / G);
+    if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
+      const int hq = head * G + crow % G;
+      const int64_t prow = ((int64_t)s * p.heads + hq) * p.num_slots + sb + chunk;
+      float* dst = p.o_part + prow * D + ccol;
+#pragma unroll
+      for (int c = 0; c < D / 16; c += 4) {
+        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w)
+          o += *(const f32x4*)(cbuf + (w * 16 + crow) * OROW + ccol + c) * wgt[w];
+        *(f32x4*)(dst + c) = o * inv;
+      }
+      if ((tid & 15) == 0)
+        p.lse_part[prow] = (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f;
     }
   }
 }
 
-namespace {
-using SplitFn = void (*)(const SplitParams);
-template <typename T, int D>
-SplitFn split_for(int tiles) {
-  switch (tiles) {
-    case 1: return pat_split_kernel<T, D, 1>;
-    case 2: return pat_split_kernel<T, D, 2>;
-    default: return pat_split_kernel<T, D, 4>;
-  }
-}
-}  // namespace
-
-// Host launcher: picks the instance for (element type, head_dim, row tiles of 16).
-hipError_t launch_split(bool bf16, int head_dim, int row_tiles, unsigned workgroups, hipStream_t stream,
+// Host launcher: picks the instance for (element type, head_dim).
+hipError_t launch_split(bool bf16, int head_dim, unsigned workgroups, hipStream_t stream,
                         const SplitParams& params) {
-  SplitFn fn;
-  if (bf16) fn = head_dim == 64 ? split_for<__bf16, 64>(row_tiles) : split_for<__bf16, 128>(row_tiles);
-  else fn = head_dim == 64 ? split_for<_Float16, 64>(row_tiles) : split_for<_Float16, 128>(row_tiles);
+  void (*fn)(const SplitParams);
+  if (bf16) fn = head_dim == 64 ? pat_split_kernel<__bf16, 64> : pat_split_kernel<__bf16, 128>;
+  else fn = head_dim == 64 ? pat_split_kernel<_Float16, 64> : pat_split_kernel<_Float16, 128>;
   hipLaunchKernelGGL(fn, dim3(workgroups), dim3(kThreads), 0, stream, params);
   return hipGetLastError();
 }

@@ -326,6 +326,7 @@ void RadixPlanner::bucketize(const std::vector<Box>& boxes,
   }
 
   Plan plan;
+  std::vector<int32_t> boxes_seen(split_per_seq_.size(), 0);  // per sequence, boxes emitted so far
   for (const auto& mnw : buckets) {
     const auto& members = grouped[mnw];
     if (members.empty()) continue;
@@ -337,11 +338,14 @@ void RadixPlanner::bucketize(const std::vector<Box>& boxes,
     }
     bk.q_table.assign(members.size() * (size_t)bk.max_seqs, 0);
     bk.block_table.assign(members.size() * (size_t)bk.max_blocks, 0);
+    bk.q_slot.assign(members.size() * (size_t)bk.max_seqs, 0);
     for (size_t r = 0; r < members.size(); ++r) {
       const Box& b = boxes[members[r]];
       std::copy(b.seqs.begin(), b.seqs.end(), bk.q_table.begin() + (std::ptrdiff_t)(r * bk.max_seqs));
       std::copy(b.blocks.begin(), b.blocks.end(),
                 bk.block_table.begin() + (std::ptrdiff_t)(r * bk.max_blocks));
+      for (size_t j = 0; j < b.seqs.size(); ++j)
+        bk.q_slot[r * (size_t)bk.max_seqs + j] = boxes_seen.at((size_t)b.seqs[j])++;
       bk.q_len.push_back((int32_t)b.seqs.size());
       bk.block_len.push_back((int32_t)b.blocks.size());
       bk.num_seqs.push_back(b.num_seqs);
@@ -371,6 +375,7 @@ void RadixPlanner::bucketize(const std::vector<Box>& boxes,
     v.num_seqs = bk.num_seqs.data();
     v.rank = bk.rank.data();
     v.kv = bk.kv.data();
+    v.q_slot = bk.q_slot.data();
     plan.views.push_back(v);
   }
   plan.valid = true;
@@ -386,6 +391,7 @@ void RadixPlanner::bucketize(const std::vector<Box>& boxes,
     v.num_seqs = bk.num_seqs.data();
     v.rank = bk.rank.data();
     v.kv = bk.kv.data();
+    v.q_slot = bk.q_slot.data();
   }
 }
 

@@ -63,6 +63,7 @@ struct Bucket {
   int32_t mnw[3];
   int32_t max_seqs = 0, max_blocks = 0;
   std::vector<int32_t> q_table, block_table;  // padded, row-major
+  std::vector<int32_t> q_slot;                // padded like q_table
   std::vector<int32_t> q_len, block_len, num_seqs, rank, kv;
 };
 

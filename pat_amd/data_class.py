@@ -170,6 +170,10 @@ class KernelInfo:
     max_blocks_in_CTA: int = 0
     reverse_index: Any = None
     sort_index: Any = None
+    # Not in the reference: per bucket, for every (box, sequence) the box's ordinal among the
+    # boxes of that sequence. Passing it to prefix_attn_with_kvcache(..., slot_tables=...) files
+    # partial results by this ordinal instead of by CTA_rank.
+    slot_tables: Any = field(default_factory=list)
 
     def to_tensor(self, device) -> None:
         def vectors(cols: Iterable) -> list:
@@ -194,6 +198,8 @@ class KernelInfo:
             self.q_tables = matrices(self.q_tables)
         if not all(isinstance(t, torch.Tensor) for t in self.block_tables):
             self.block_tables = matrices(self.block_tables)
+        if self.slot_tables and not all(isinstance(t, torch.Tensor) for t in self.slot_tables):
+            self.slot_tables = matrices(self.slot_tables)
 
 
 def create_seq_group(block_tables: List[List[int]], seq_lens: List[int], block_size: int) -> SeqGroup:

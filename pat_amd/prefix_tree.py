@@ -49,6 +49,8 @@ def plan_to_kernel_info(view: _lib.PlanView) -> KernelInfo:
         ki.num_seqs_per_CTAs.append(_copy(bk.num_seqs, n))
         ki.CTA_ranks.append(_copy(bk.rank, n))
         ki.kv_in_CTAs.append(_copy(bk.kv, n))
+        sl = np.ctypeslib.as_array(bk.q_slot, shape=(n, ws)) if ws else np.zeros((n, 0), np.int32)
+        ki.slot_tables.append([sl[i, :ql[i]].tolist() for i in range(n)])
     ki.num_split_per_seq = _copy(view.num_split_per_seq, view.batch)
     ki.max_split_per_seq = view.max_split_per_seq
     ki.max_seqs_in_CTA = view.max_seqs_in_box

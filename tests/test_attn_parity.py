@@ -1,0 +1,208 @@
+"""GPU parity: the HIP path (through the C ABI of libpat_amd) against the CPU attention oracle
+on the same seeded inputs.
+
+Tolerances: max-abs 2e-3 for fp16 and 1.6e-2 for bf16 outputs (fp32 accumulation on both
+sides), LSE within 1e-4 relative.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import attn_oracle as ao
+from pat_amd import PrefixTree, PrefixTreeCPP, prefix_attn_with_kvcache, workloads
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
+LSE_RTOL = 1e-4
+
+
+def _device():
+    assert torch.cuda.is_available(), "GPU tests need an AMD GPU"
+    return torch.device("cuda:0")
+
+
+def _oracle(w, q, k, v):
+    return ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, w.seq_lens)
+
+
+def _assert_close(name, out, lse, ref_out, ref_lse, dtype):
+    err = (out.float().cpu() - ref_out.float()).abs().max().item()
+    lerr = ((lse.cpu() - ref_lse).abs() / ref_lse.abs().clamp_min(1.0)).max().item()
+    print(f"[parity] {name}: max|out - ref| = {err:.3e} (tol {TOL[dtype]:.1e}), LSE rel = {lerr:.3e}", flush=True)
+    assert err <= TOL[dtype], f"{name}: output error {err}"
+    assert lerr <= LSE_RTOL, f"{name}: LSE error {lerr}"
+
+
+def _run_tree(w, q, k, v, chunk_env=None):
+    dev = q.device
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    return out, lse
+
+
+@pytest.mark.parametrize("name", workloads.NAMES)
+def test_workload_tree_overload(name):
+    print(f"[case] workload {name} tree overload", flush=True)
+    dev = _device()
+    w = workloads.make(name, seed=0)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(name, out, lse, ref_out, ref_lse, w.dtype)
+
+
+@pytest.mark.parametrize("name,dtype", [("c1", torch.float16), ("c1", torch.bfloat16), ("c2", torch.float16),
+                                        ("c4", torch.bfloat16)])
+def test_workload_table_overload(name, dtype):
+    # the benchmark's call form: Python PrefixTree + KernelInfo.to_tensor + positional tables
+    print(f"[case] workload {name} table overload {dtype}", flush=True)
+    dev = _device()
+    w = workloads.make(name, seed=2)
+    w.dtype = dtype
+    q, k, v = w.tensors(dev)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+    ki.to_tensor(device=dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                             ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                             ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, None, softmax_lse=lse,
+                             slot_tables=ki.slot_tables if name == "c4" else None)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"{name}/{dtype}", out, lse, ref_out, ref_lse, dtype)
+
+
+def test_manual_fixture_partial_pages():
+    # the reference's manual fixture (test/test.py:233-239): 33-token requests, partly filled last pages
+    print("[case] manual fixture", flush=True)
+    dev = _device()
+    w = workloads.Workload("manual", 32, 8, 128, torch.float16, 16, [33, 33, 33], [[0, 1, 5], [0, 2, 6], [3, 4, 7]],
+                           13, 0, 0)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("manual", out, lse, ref_out, ref_lse, torch.float16)
+
+
+@pytest.mark.parametrize("spec,heads", [("1,4,16_32,256,32", (64, 8)), ("1,8_640,32", (64, 8)),
+                                        ("1,2,4,8,16,32,64_32,512,32,256,32,32,32", (64, 8)),
+                                        ("4,16_4096,256", (32, 32)), ("1,10_4096,416", (16, 8))])
+def test_reference_tree_specs_page32(spec, heads):
+    # tree batches of the reference's own test (test/test.py:174-187): page 32, fp16, d 128
+    print(f"[case] tree spec {spec} heads {heads}", flush=True)
+    import random
+    from pat_amd import generate_tree_seqs
+    dev = _device()
+    random.seed(11)
+    group, nblk = generate_tree_seqs(spec, 32)
+    w = workloads.Workload(spec, heads[0], heads[1], 128, torch.float16, 32, group.seqlens, group.get_block_ids(),
+                           nblk, 0, 4)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(spec, out, lse, ref_out, ref_lse, torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d,heads", [(64, (8, 8)), (64, (16, 2)), (128, (8, 4)), (128, (16, 8))])
+def test_ragged_random_forest(dtype, d, heads):
+    print(f"[case] ragged forest d={d} heads={heads} {dtype}", flush=True)
+    import random
+    dev = _device()
+    r = random.Random(d + heads[0])
+    rows, lens, nxt = [], [], 0
+    for _ in range(37):
+        row = []
+        if rows and r.random() < 0.8:
+            base = rows[r.randrange(len(rows))]
+            row = list(base[:r.randint(0, len(base) - 1)])
+        extra = r.randint(1, 40)
+        row += list(range(nxt, nxt + extra)); nxt += extra
+        rows.append(row)
+        lens.append(len(row) * 16 - r.randint(0, 15))
+    perm = list(range(nxt)); r.shuffle(perm)
+    rows = [[perm[x] for x in row] for row in rows]
+    # on such forests the reference scheduler can hand one rank to two boxes of a request; the
+    # tree form files partial results by box ordinal, so the result is right all the same
+    w = workloads.Workload("forest", heads[0], heads[1], d, dtype, 16, lens, rows, nxt, 0, 9)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("forest", out, lse, ref_out, ref_lse, dtype)
+
+
+def test_strided_views_and_output_in_place():
+    # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
+    print("[case] strided views", flush=True)
+    dev = _device()
+    w = workloads.make("c1", seed=4)
+    q, k, v = w.tensors(dev)
+    kv = torch.stack([k, v])                      # [2, blocks, page, h, d]
+    qbig = torch.zeros(w.batch + 3, w.heads, w.head_dim + 64, dtype=q.dtype, device=dev)
+    qbig[3:, :, :w.head_dim] = q[:, 0]
+    qv = qbig[3:, :, :w.head_dim].unsqueeze(1)
+    obig = torch.zeros(w.batch + 5, w.heads, w.head_dim, dtype=q.dtype, device=dev)
+    ov = obig[5:].unsqueeze(1)
+    tree = PrefixTreeCPP(16)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, 1, 8)
+    tree.kernel_info.to_gpu(dev)
+    prefix_attn_with_kvcache(q=qv, k_cache_paged=kv[0], v_cache_paged=kv[1], tree=tree,
+                             softmax_scale=0.125, out=ov)
+    torch.cuda.synchronize()
+    ref_out, _ = _oracle(w, q, k, v)
+    assert (obig[5:].float().cpu() - ref_out[:, 0].float()).abs().max().item() <= 2e-3
+    assert obig[:5].abs().max().item() == 0
+
+
+def test_oblivious_plan_same_result_and_linearity():
+    # size-independent properties at the headline size: (1) the prefix-oblivious plan gives the same
+    # answer as the prefix-aware one; (2) attention is linear in V
+    print("[case] c2 oblivious + linearity", flush=True)
+    dev = _device()
+    w = workloads.make("c2", seed=0)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ob = workloads.oblivious_plan(w, dev)
+    out2 = torch.empty_like(q)
+    lse2 = torch.empty_like(lse)
+    prefix_attn_with_kvcache(q, k, v, ob["num_split_per_seq"], ob["query_tables"], ob["block_tables"],
+                             ob["num_seqs_per_CTAs"], ob["CTA_ranks"], ob["kv_in_CTAs"], ob["MNW"],
+                             ob["max_split_per_seq"], ob["max_seqs_in_CTA"], ob["max_blocks_in_CTA"],
+                             1.0 / math.sqrt(w.head_dim), out2, softmax_lse=lse2)
+    torch.cuda.synchronize()
+    assert (out.float() - out2.float()).abs().max().item() <= 1.6e-2
+    assert ((lse - lse2).abs() / lse.abs().clamp_min(1)).max().item() <= 1e-4
+    out3, _ = _run_tree(w, q, k, (v.float() * 2).to(v.dtype))
+    assert (out3.float() - 2 * out.float()).abs().max().item() <= 3.2e-2
+
+
+def test_validation_errors_on_gpu_tensors():
+    dev = _device()
+    w = workloads.make("c1")
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(16)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, 1, 8)
+    out = torch.empty_like(q)
+    with pytest.raises(RuntimeError, match="must be on CUDA"):
+        prefix_attn_with_kvcache(q, k, v, tree, 0.125, out)          # plan still on the CPU
+    tree.kernel_info.to_gpu(dev)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        prefix_attn_with_kvcache(q, k.to(torch.bfloat16), v, tree, 0.125, out)
+    with pytest.raises(RuntimeError, match="contiguous last dimension"):
+        prefix_attn_with_kvcache(q.transpose(2, 3).contiguous().transpose(2, 3), k, v, tree, 0.125, out)
+    with pytest.raises(RuntimeError, match="64 / 128"):
+        prefix_attn_with_kvcache(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), tree,
+                                 0.125, out[..., :32].contiguous())

@@ -1,0 +1,125 @@
+"""libpat_amd loads, exports every symbol include/pat_amd.h declares, and its GPU-free entry
+points (argument validation, launch geometry, workspace size) behave. No kernel is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from pat_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "pat_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pat_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(lib, name), f"libpat_amd.so does not export {name}"
+    assert sorted(_lib.SYMBOLS) == names       # the ctypes table covers the header, no more, no less
+    assert lib.pat_abi_version() == 1
+
+
+def _args(**over):
+    """A well-formed pat_fwd_args with fake (never dereferenced) device addresses."""
+    fake = 0x10000
+    b = (_lib.FwdBucket * 2)()
+    for i, (m, boxes, seqs, blocks) in enumerate([(64, 4, 16, 128), (16, 64, 1, 32)]):
+        b[i].q_table = b[i].block_table = b[i].num_seqs = b[i].rank = b[i].kv = fake
+        b[i].q_table_stride, b[i].block_table_stride = seqs, blocks
+        b[i].num_boxes, b[i].max_seqs, b[i].max_blocks = boxes, seqs, blocks
+        b[i].mnw[0], b[i].mnw[1], b[i].mnw[2] = m, 128, 4 if m == 64 else 1
+    a = _lib.FwdArgs()
+    a.dtype, a.batch, a.seqlen_q, a.heads, a.kv_heads = _lib.PAT_DTYPE_BF16, 64, 1, 32, 8
+    a.head_dim, a.page_size, a.num_pages = 128, 16, 4096
+    a.q = a.k = a.v = a.out = a.num_split_per_seq = fake
+    a.q_stride = (C.c_int64 * 3)(4096, 4096, 128)
+    a.k_stride = (C.c_int64 * 3)(16 * 8 * 128, 8 * 128, 128)
+    a.v_stride = (C.c_int64 * 3)(16 * 8 * 128, 8 * 128, 128)
+    a.o_stride = (C.c_int64 * 3)(4096, 4096, 128)
+    a.max_split_per_seq, a.max_seqs_in_box, a.max_blocks_in_box = 2, 16, 128
+    a.softmax_scale = 0.088
+    a.num_buckets, a.buckets = 2, C.cast(b, C.POINTER(_lib.FwdBucket))
+    a._keep = b
+    for k, v in over.items():
+        setattr(a, k, v)
+    return a
+
+
+def test_validate_accepts_headline_shape():
+    lib = _lib.load()
+    assert lib.pat_fwd_validate(C.byref(_args())) == 0
+
+
+@pytest.mark.parametrize("field,value,needle", [
+    ("dtype", 7, "only support fp16 and bf16"),
+    ("max_split_per_seq", 33, "only supports up to 32 splits"),
+    ("max_split_per_seq", 0, "no case that a seq has no block"),
+    ("head_dim", 96, "head_size_og must be 64 / 128"),
+    ("page_size", 24, "divisible by 16"),
+    ("kv_heads", 5, "must divide number of heads"),
+    ("kv_heads", 2, "hq/hkv = 1, 2, 4, 8"),
+    ("batch", 0, "batch size must be positive"),
+    ("seqlen_q", 2, "decode only"),
+    ("q", 0, "non-null"),
+    ("num_buckets", 13, "between 1 and 12"),
+])
+def test_validate_rejects(field, value, needle):
+    lib = _lib.load()
+    rc = lib.pat_fwd_validate(C.byref(_args(**{field: value})))
+    assert rc == _lib.PAT_ERR_INVALID
+    assert needle in _lib.last_error()
+    with pytest.raises(RuntimeError):
+        _lib.check(rc)
+
+
+def test_validate_rejects_bad_bucket_and_strides():
+    lib = _lib.load()
+    a = _args()
+    a.buckets[0].mnw[0] = 48
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "tile_q" in _lib.last_error()
+    a = _args()
+    a.k_stride = (C.c_int64 * 3)(16 * 8 * 128 + 4, 8 * 128, 128)
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "multiples of 8" in _lib.last_error()
+    a = _args()
+    a.buckets[1].max_seqs = 32      # 32 sequences x 4 heads per kv head > 64 rows
+    a.buckets[1].q_table_stride = 32
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "64 rows" in _lib.last_error()
+
+
+def test_geometry_and_workspace_are_consistent():
+    lib = _lib.load()
+    a = _args()
+    g = _lib.FwdGeometry()
+    assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
+    assert g.chunk_tokens % 32 == 0 and g.tall_chunk_tokens % 32 == 0
+    assert g.chunks_per_rank == max(-(-128 * 16 // g.tall_chunk_tokens), -(-32 * 16 // g.chunk_tokens))
+    assert g.num_slots == g.chunks_per_rank * 2
+    assert g.num_workgroups == 8 * (4 * -(-128 * 16 // g.tall_chunk_tokens) + 64 * -(-32 * 16 // g.chunk_tokens))
+    need = C.c_size_t()
+    assert lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)) == 0
+    rows = 64 * 32 * g.num_slots
+    assert need.value >= rows * 128 * 4 + rows * 4
+    # launching without a workspace is refused before any GPU call
+    a.workspace, a.workspace_bytes = 0, 0
+    assert lib.pat_fwd_launch(C.byref(a), None) == _lib.PAT_ERR_WORKSPACE
+
+
+def test_tree_handles_and_errors():
+    lib = _lib.load()
+    h = C.c_void_p()
+    assert lib.pat_tree_create(0, C.byref(h)) == _lib.PAT_ERR_INVALID
+    assert lib.pat_tree_create(16, C.byref(h)) == 0
+    view = _lib.PlanView()
+    assert lib.pat_tree_plan(h, C.byref(view)) == _lib.PAT_ERR_INVALID and "no plan" in _lib.last_error()
+    assert lib.pat_tree_num_nodes(h) == 1
+    nv = _lib.NodeView()
+    assert lib.pat_tree_node(h, 5, C.byref(nv)) == _lib.PAT_ERR_INDEX
+    lib.pat_tree_destroy(h)
