@@ -23,6 +23,10 @@ namespace {
 
 constexpr int kNumCUs = 256;        // MI355X
 constexpr int kMaxChunksPerRank = 64;
+constexpr int kTargetWgsPerCU = 2;  // what fits at once: 2 workgroups of 4 waves per CU at head_dim 128
+constexpr int kMinChunk = 128;      // tokens
+constexpr int kMaxChunk = 2048;
+constexpr int kTallChunk = 256;
 
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
@@ -76,6 +80,10 @@ int check_args(const pat_fwd_args* a) {
     for (int i = 0; i < 3; ++i)
       if (strides[t][i] % 8 != 0 || strides[t][i] < 0)
         return fail(PAT_ERR_INVALID, std::string(names[t]) + " strides must be non-negative multiples of 8 elements");
+  // lanes address rows inside a page with 32-bit byte offsets
+  if (a->k_stride[1] * (int64_t)a->page_size >= (int64_t(1) << 29) ||
+      a->v_stride[1] * (int64_t)a->page_size >= (int64_t(1) << 29))
+    return fail(PAT_ERR_INVALID, "k_cache_paged / v_cache_paged: a block must span less than 1 GiB");
   const void* ptrs[3] = {a->q, a->k, a->v};
   for (int t = 0; t < 3; ++t)
     if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0)
@@ -104,44 +112,46 @@ int check_args(const pat_fwd_args* a) {
   return PAT_OK;
 }
 
-// Launch geometry. A workgroup streams one chunk of one box for one kv head; a bucket reserves
-// ceil(widest box / chunk) workgroups per box (those past a box's real length exit at once).
+// Launch geometry. A workgroup streams one chunk of one box's KV for one kv head; a bucket
+// reserves ceil(widest box / chunk) workgroups per (box, head), those past a box's real length
+// exit at once.
 //  * boxes of <= 16 rows split the chunk's 32-token steps over the 4 waves: the chunk is sized
-//    so that the device sees a few workgroups per CU, between 128 and 1024 tokens;
-//  * boxes of 17..64 rows give every wave the whole chunk (rows are split instead) and write
-//    16 KB..32 KB of partial output per workgroup, so they use a fixed, longer chunk.
-// PAT_CHUNK_TOKENS / PAT_TALL_CHUNK_TOKENS override both (tuning aid).
+//    so that this work fills the device with about kTargetWgsPerCU workgroups per CU - few
+//    enough that all are resident at once, so every CU has loads in flight from start to end;
+//  * boxes of 17..64 rows walk the chunk step by step with all 4 waves (one row tile each) and
+//    write 16..32 KB of partial output per workgroup: they get a fixed chunk.
+// PAT_CHUNK_TOKENS / PAT_TALL_CHUNK_TOKENS override the two sizes (tuning aid).
 int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   const int page = a->page_size;
   const int64_t unit = (int64_t)page * kStepTokens / gcd64(page, kStepTokens);  // lcm(page, 32)
   auto round_unit = [&](int64_t c) { return std::max<int64_t>(unit, ceil_div64(c, unit) * unit); };
-  int64_t short_total = 0;
+  const int64_t cap = (int64_t)kMaxChunkPages * page / unit * unit;  // page ids of a chunk sit in 2 VGPRs
+  if (cap <= 0) return fail(PAT_ERR_INVALID, "page size too large for one workgroup");
+  int64_t work = 0;
   for (int i = 0; i < a->num_buckets; ++i)
     if (row_tiles(a->buckets[i].mnw[0]) == 1)
-      short_total += (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
+      work += (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
   int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
   if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
-  if (chunk <= 0) chunk = std::max<int64_t>(128, std::min<int64_t>(1024, short_total / (4 * kNumCUs)));
-  if (tall <= 0) tall = 256;
-  const int64_t cap = (int64_t)kMaxChunkPages * page / unit * unit;  // page ids of a chunk sit in LDS
-  if (cap <= 0) return fail(PAT_ERR_INVALID, "page size too large for one workgroup");
+  if (chunk <= 0) chunk = std::max<int64_t>(kMinChunk, std::min<int64_t>(kMaxChunk, work / (kTargetWgsPerCU * kNumCUs)));
+  if (tall <= 0) tall = kTallChunk;
+  g->chunk = (int)std::min(round_unit(chunk), cap);
+  g->tall_chunk = (int)std::min(round_unit(tall), cap);
   g->chunks_per_rank = 1;
   g->total_wgs = 0;
   for (int i = 0; i < a->num_buckets; ++i) {
-    const bool is_tall = row_tiles(a->buckets[i].mnw[0]) > 1;
     const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-    int64_t c = round_unit(is_tall ? tall : chunk);
-    while (ceil_div64(tok, c) > kMaxChunksPerRank) c += unit;   // bounded slots per box
-    if (c > cap) return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
+    int64_t c = row_tiles(a->buckets[i].mnw[0]) > 1 ? g->tall_chunk : g->chunk;
+    while (ceil_div64(tok, c) > kMaxChunksPerRank && c + unit <= cap) c += unit;   // bounded slots per box
+    if (ceil_div64(tok, c) > kMaxChunksPerRank)
+      return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
     const int n = (int)std::max<int64_t>(1, ceil_div64(tok, c));
     g->bucket_chunk[i] = (int)c;
     g->bucket_chunks[i] = n;
     g->chunks_per_rank = std::max(g->chunks_per_rank, n);
     g->total_wgs += (int64_t)a->buckets[i].num_boxes * n * a->kv_heads;
   }
-  g->chunk = (int)round_unit(chunk);
-  g->tall_chunk = (int)round_unit(tall);
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
   if (g->total_wgs > INT32_MAX) return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   return PAT_OK;
@@ -239,6 +249,12 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
     }
     sp.num_buckets = nb;
     sp.total_wgs = (int32_t)wg;
+#ifdef PAT_TRACE
+    sp.trace = nullptr;
+    if (const char* env = std::getenv("PAT_TRACE_PTR")) sp.trace = reinterpret_cast<long long*>(std::strtoull(env, nullptr, 0));
+    sp.debug_mode = 0;
+    if (const char* env = std::getenv("PAT_DEBUG_MODE")) sp.debug_mode = std::atoi(env);
+#endif
     if (wg > 0) {
       const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, (unsigned)wg, stream, sp);
       if (e != hipSuccess) return hip_fail(e, "split kernel launch");

@@ -8,7 +8,7 @@ constexpr int kMaxBuckets = 12;    // the reference dispatches 12 tile shapes (s
 constexpr int kWaves = 4;          // waves per split-kernel workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kStepTokens = 32;    // KV tokens one wave consumes per loop iteration
-constexpr int kMaxChunkPages = 128; // page ids one workgroup stages in LDS
+constexpr int kMaxChunkPages = 128; // page ids of a chunk: two per lane of a wave
 
 // One tile bucket as the split kernel sees it.
 struct BucketDev {
@@ -26,7 +26,7 @@ struct BucketDev {
   int32_t chunk_tokens;  // KV tokens per workgroup (multiple of 32 and of page_size)
   int32_t chunks;        // workgroups along the KV axis reserved per box
   int32_t wg_begin;      // first workgroup of this bucket
-  int32_t row_tiles;     // 1: boxes of <= 16 rows (KV steps split over waves); >1: rows split over waves
+  int32_t row_tiles;     // 16-row tiles per box: 1 = KV steps split over waves, 2/4 = one wave per tile
   int32_t pad_;
 };
 
@@ -47,6 +47,10 @@ struct SplitParams {
   int32_t total_wgs;
   float scale_log2;         // softmax_scale * log2(e)
   int32_t num_buckets;
+#ifdef PAT_TRACE
+  long long* trace;         // debug builds only: 8 timestamps/ids per workgroup
+  int debug_mode;           // debug builds only: 1 = loads without compute, 2 = compute without loads
+#endif
   BucketDev bucket[kMaxBuckets];
 };
 

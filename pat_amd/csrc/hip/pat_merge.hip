@@ -43,7 +43,8 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   const float total = (sum > 0.f) ? mx + logf(sum) : -__builtin_inff();
 
-  // pass 2: weighted sum of the filled slots
+  // pass 2: weighted sum of the filled slots, 8 at a time so that their loads overlap
+  constexpr int kBatch = 8;
   float acc[CPL];
 #pragma unroll
   for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
@@ -53,16 +54,33 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
     const float w_mine = (mine > -__builtin_inff()) ? __expf(mine - total) : 0.f;
     unsigned long long live = __ballot(w_mine > 0.f);
     while (live) {
-      const int j = __builtin_ctzll(live);
-      live &= live - 1;
-      const float w = __shfl(w_mine, j);
-      const float* row = op + (int64_t)(base + j) * D + lane * CPL;
-      if (CPL == 2) {
-        const float2 v = *(const float2*)row;
-        acc[0] += w * v.x;
-        acc[CPL - 1] += w * v.y;
-      } else {
-        acc[0] += w * row[0];
+      int js[kBatch];
+      float v[kBatch][CPL];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        js[b] = live ? __builtin_ctzll(live) : -1;
+        live &= live - 1;   // 0 stays 0
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        if (js[b] >= 0) {
+          const float* row = op + (int64_t)(base + js[b]) * D + lane * CPL;
+          if (CPL == 2) {
+            const float2 t = *(const float2*)row;
+            v[b][0] = t.x;
+            v[b][CPL - 1] = t.y;
+          } else {
+            v[b][0] = row[0];
+          }
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        if (js[b] >= 0) {
+          const float w = __shfl(w_mine, js[b]);
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) acc[c] += w * v[b][c];
+        }
       }
     }
   }

@@ -1,5 +1,6 @@
 // Split-KV forward kernel for gfx950 (MI355X): one workgroup streams one chunk of one
-// packed box's KV for one kv-head and writes a normalised partial output + LSE.
+// packed box's KV for one kv-head and one 16-row tile of the box, and writes a normalised
+// partial output + LSE per row.
 //
 // Functional contract (what the reference's pat_fwd_splitkv_kernel computes,
 // csrc/pat_fwd_kernel.h:25-299): rows r = g + G*j of a box are (sequence
@@ -8,21 +9,25 @@
 // those tokens plus LSE = max + ln(sum) (csrc/softmax.h:169-188).
 //
 // Mapping to the hardware (this kernel's own design):
-//  * a workgroup = 4 wave64 working on one (box, kv-head, chunk) in one of two ways:
-//      - boxes of up to 16 rows: each wave owns every 4th 32-token step of the chunk and
-//        runs an independent online softmax; the 4 states are combined through LDS;
-//      - boxes of 17..64 rows: wave w owns rows 16w..16w+15 over the whole chunk (the
-//        waves re-read the same K/V lines through L1), no combine needed.
-//    Either way one (box, head, chunk) yields one partial row set, every wave carries a
-//    single 16-row tile of state, and one launch covers all buckets.
-//  * S^T = K.Q^T on v_mfma_f32_16x16x32: K rows are the MFMA A operand, so a lane
-//    loads 16 contiguous bytes of one token straight from HBM into operand layout
-//    (no LDS for K). The accumulator layout of S^T is the B-operand layout of
+//  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each. The kv-head is the
+//    fastest-varying part of the workgroup index: workgroups are dealt to the 8 XCDs
+//    round-robin, so with 8 kv-heads XCD x serves head x and boxes that share KV pages (the
+//    boxes of one prefix node) find them in that XCD's L2.
+//  * boxes of up to 16 rows (one MFMA row tile): each wave owns every 4th 32-token step of
+//    the chunk on wave-private tiles and runs an independent online softmax; the 4 states are
+//    combined through LDS at the end. K rows are the MFMA A operand of S^T = K.Q^T, so a lane
+//    loads 16 contiguous bytes of one token straight from HBM into operand layout (no LDS).
+//  * boxes of 17..64 rows: wave w owns rows 16w..16w+15 and all waves walk the same steps;
+//    each step's K and V tile is fetched once per workgroup (coalesced 256-byte rows, 4 steps
+//    ahead), shared through a two-stage LDS buffer and read as operands from there.
+//  * S^T on v_mfma_f32_16x16x32; its accumulator layout is the B-operand layout of
 //    O^T = V^T.P^T, so P never moves between lanes.
-//  * V must be contracted along tokens but is contiguous along head_dim: each wave
-//    stages its 32 x D tile in a private, padded LDS region (16-byte writes) and
-//    reads it back transposed with ds_read_b64_tr_b16.
+//  * V must be contracted along tokens but is contiguous along head_dim: V tiles sit row-major
+//    in padded LDS rows and are read back transposed with ds_read_b64_tr_b16.
 //  * all softmax state of a row lives in the 4 lanes {n, n+16, n+32, n+48}.
+//  * the chunk's page ids live in two VGPRs per wave (lane i holds page i) and are
+//    broadcast with v_readlane, so the prologue is two dependent memory round trips:
+//    {plan scalars, page ids, sequence ids} -> {K, V, Q}.
 #include <hip/hip_runtime.h>
 
 #include "fwd_params.hpp"
@@ -56,31 +61,42 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 
 template <typename T, int D>
-__global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p) {
+__global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   constexpr int KK = D / 32;             // MFMA k-steps across head_dim in S^T = K.Q^T
   constexpr int DB = D / 16;             // 16-wide head_dim blocks of O^T
-  constexpr int NV = D / 16;             // 16-byte V loads per lane per 32-token step
+  constexpr int NV = D / 16;             // 16-byte V loads per lane per step (wave-private tiles)
+  constexpr int NP = D / 64;             // 16-byte K (and V) loads per thread per step (shared tiles)
+  constexpr int PF = 2;                  // shared tiles: steps kept in flight per workgroup
   constexpr int CPR = D / 8;             // 16-byte pieces per token row
-  constexpr int RS = D * 2 + 32;         // padded LDS row stride of the V tile, bytes
-  constexpr int VSTAGE = kStepTokens * RS;
+  constexpr int TPL = 64 / CPR;          // tokens covered by one wave-wide load instruction
+  constexpr int RSK = D * 2 + 16;        // LDS row stride of a K tile (conflict-free 16-byte row reads)
+  constexpr int RSV = D * 2 + 32;        // LDS row stride of a V tile (conflict-free transposed reads)
+  constexpr int VSTAGE = kStepTokens * RSV;            // one wave's private V tile
+  constexpr int SHARED = kStepTokens * (RSK + RSV);    // one shared K + V stage
   constexpr int OROW = D + 4;            // padded row of the combine buffer, floats
   constexpr int COMBINE = kWaves * 16 * OROW * 4;
-  constexpr int SMEM = (kWaves * VSTAGE > COMBINE) ? kWaves * VSTAGE : COMBINE;
+  constexpr int SMEM0 = (kWaves * VSTAGE > COMBINE) ? kWaves * VSTAGE : COMBINE;
+  constexpr int SMEM = (SMEM0 > 2 * SHARED) ? SMEM0 : 2 * SHARED;
 
   __shared__ __attribute__((aligned(16))) char smem[SMEM];
-  __shared__ int s_pages[kMaxChunkPages];
   __shared__ float s_m[kWaves][16];
   __shared__ float s_l[kWaves][16];
 
+#ifdef PAT_TRACE
+  long long tr[6] = {wall_clock64(), 0, 0, 0, 0, 0};
+#define PAT_STAMP(i) tr[i] = wall_clock64()
+#else
+#define PAT_STAMP(i)
+#endif
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int g = lane >> 4;   // lane group 0..3
   const int n = lane & 15;   // index inside the group
 
-  // ---- which (bucket, box, chunk, kv-head) is this workgroup? -----------------
+  // ---- which (bucket, box, chunk, kv-head) is this workgroup? ---------------------------
   const int wg = blockIdx.x;
   int bi = 0;
   for (int i = 1; i < p.num_buckets; ++i)
@@ -93,113 +109,108 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
   const int box = local / bk.chunks;
   if (box >= bk.num_boxes) return;
 
+  // Boxes of up to 16 rows: the 4 waves split the chunk's steps, each on wave-private tiles.
+  // Taller boxes: wave w owns rows 16w..16w+15, all waves walk the same steps on tiles shared
+  // through LDS.
+  const bool shared_tiles = bk.row_tiles > 1;
   const int G = p.group;
-  const int rank = bk.rank[box];
-  int nseq = bk.num_seqs[box];
-  nseq = nseq < 0 ? 0 : (nseq > bk.max_seqs ? bk.max_seqs : nseq);
-  int R = nseq * G;
-  if (R > 64) R = 64;
-  const bool tall = bk.row_tiles > 1;            // rows split across waves instead of KV steps
-  const int row0 = tall ? wave * 16 : 0;         // first row of this wave's tile
-  int kv = bk.kv[box];
-  const int kv_cap = bk.max_blocks * p.page_size;
-  kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
+  const int page = p.page_size;
+  const int row0 = shared_tiles ? wave * 16 : 0;
   const int t_begin = chunk * bk.chunk_tokens;
   const int* __restrict__ qt = bk.q_table + (int64_t)box * bk.q_stride;
-  // Partial-slot ordinal of this box per sequence: the plan's own rank, or - when the caller
-  // supplies it - the box's ordinal among the boxes of that sequence (always collision-free).
   const int* __restrict__ qs = bk.q_slot ? bk.q_slot + (int64_t)box * bk.q_stride : nullptr;
-  auto slot_base = [&](int j) -> int {
-    const int ord = qs ? qs[j] : rank;
-    return ((unsigned)ord < (unsigned)p.max_split) ? ord * p.chunks_per_rank : -1;
-  };
+  const int* __restrict__ bt = bk.block_table + (int64_t)box * bk.bt_stride;
 
-  // ---- slots of this rank nobody will fill are marked empty (-inf) -------------
+  // ---- round trip 1: everything that depends on the box index only ---------------------
+  const int rank = bk.rank[box];
+  int nseq = bk.num_seqs[box];
+  int kv = bk.kv[box];
+  // this lane's row: sequence id and partial-slot ordinal (the plan's own rank, or - when the
+  // caller supplies it - the box's ordinal among the boxes of that sequence)
+  const int my_j = (row0 + n) / G;
+  const bool j_ok = my_j < bk.max_seqs;
+  const int my_seq_raw = j_ok ? qt[my_j] : -1;
+  const int my_ord = (j_ok && qs) ? qs[my_j] : rank;
+  // page ids of the chunk: lane i of every wave holds pages i and 64 + i
+  const int first_page = t_begin / page;
+  int pg0 = (first_page + lane < bk.max_blocks) ? bt[first_page + lane] : 0;
+  int pg1 = (first_page + 64 + lane < bk.max_blocks) ? bt[first_page + 64 + lane] : 0;
+  pg0 = pg0 < 0 ? 0 : (pg0 >= p.num_pages ? p.num_pages - 1 : pg0);
+  pg1 = pg1 < 0 ? 0 : (pg1 >= p.num_pages ? p.num_pages - 1 : pg1);
+
+  nseq = nseq < 0 ? 0 : (nseq > bk.max_seqs ? bk.max_seqs : nseq);
+  int R = nseq * G;
+  const int row_cap = shared_tiles ? 64 : 16;
+  if (R > row_cap) R = row_cap;
+  const int kv_cap = bk.max_blocks * page;
+  kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
+  if (R == 0) return;
+  const bool has_rows = row0 < R;   // false: a wave that only helps loading shared tiles
+  PAT_STAMP(1);
+
+  const bool row_ok = (row0 + n < R) && ((unsigned)my_seq_raw < (unsigned)p.batch) &&
+                      ((unsigned)my_ord < (unsigned)p.max_split);
+  const int my_hq = head * G + (row0 + n) % G;
+  // first partial slot of (my row, this box); -1: the row is not to be written
+  const int64_t my_slot0 = row_ok ? ((int64_t)my_seq_raw * p.heads + my_hq) * p.num_slots +
+                                        (int64_t)my_ord * p.chunks_per_rank : -1;
+
+  // ---- slots of this box that no workgroup will fill are marked empty (-inf) ------------
   {
     const bool empty = t_begin >= kv;
     const int first = empty ? chunk : chunk + 1;
     const int last = (chunk == bk.chunks - 1) ? p.chunks_per_rank : chunk + 1;  // exclusive
-    const int nmark = last - first;
-    for (int idx = tid; idx < R * nmark; idx += kThreads) {
-      const int r = idx / nmark, c = first + idx % nmark;
-      const int s = qt[r / G];
-      const int sb = slot_base(r / G);
-      if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
-        const int hq = head * G + r % G;
-        p.lse_part[((int64_t)s * p.heads + hq) * p.num_slots + sb + c] = neg_inf();
-      }
-    }
+    if ((shared_tiles || wave == 0) && g == 0 && my_slot0 >= 0)
+      for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
     if (empty) return;
   }
   const int t_end = (kv < t_begin + bk.chunk_tokens) ? kv : t_begin + bk.chunk_tokens;
+  const int last_rel = t_end - t_begin - 1;
+  const int nsteps = (t_end - t_begin + kStepTokens - 1) / kStepTokens;
 
-  // ---- page ids of the chunk -> LDS ---------------------------------------------
-  const int page = p.page_size;
-  {
-    const int* __restrict__ bt = bk.block_table + (int64_t)box * bk.bt_stride;
-    const int first_page = t_begin / page;
-    const int npages = (t_end - t_begin + page - 1) / page;
-    for (int i = tid; i < npages; i += kThreads) {
-      int pg = bt[first_page + i];
-      pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
-      s_pages[i] = pg;
-    }
-  }
+  // ---- addressing ---------------------------------------------------------------------------
+  // A 16-token half of a step never straddles a page, so its rows share one base address that is
+  // uniform over the wave (page id broadcast with v_readlane, 64-bit arithmetic on the scalar
+  // unit) and every lane adds a 32-bit byte offset that does not change from step to step.
+  const int hpp = page >> 4;                                   // halves per page
+  const int hshift = ((hpp & (hpp - 1)) == 0) ? 31 - __builtin_clz(hpp) : -1;
+  const int64_t ksp = p.k_stride_page * (int64_t)sizeof(T), kss = p.k_stride_slot * (int64_t)sizeof(T);
+  const int64_t vsp = p.v_stride_page * (int64_t)sizeof(T), vss = p.v_stride_slot * (int64_t)sizeof(T);
+  const char* __restrict__ kbase = (const char*)p.k + (int64_t)head * p.k_stride_h * (int64_t)sizeof(T);
+  const char* __restrict__ vbase = (const char*)p.v + (int64_t)head * p.v_stride_h * (int64_t)sizeof(T);
+  const int ntok = t_end - t_begin;
 
-  // ---- Q rows as MFMA B operand (lane (g, n): row row0 + n, dims kk*32 + g*8 .. +7) ----
+  // base address of half h (chunk-relative, uniform, h*16 < ntok)
+  auto half_base = [&](const char* base, int64_t sp, int64_t ss, int h) -> const char* {
+    int pidx, s16;
+    if (hshift >= 0) { pidx = h >> hshift; s16 = h & (hpp - 1); }
+    else { pidx = h / hpp; s16 = h - pidx * hpp; }
+    const int pg = __builtin_amdgcn_readlane(pidx < 64 ? pg0 : pg1, pidx & 63);
+    return base + (int64_t)pg * sp + (int64_t)(s16 * 16) * ss;
+  };
+  // per-lane address of token tok (chunk-relative; clamped to the last valid token, whose score
+  // is masked and whose probability is 0 wherever it stands in for a token past the end). Only
+  // the last, partial step of a chunk takes this slower route.
+  auto lane_row = [&](const char* base, int64_t sp, int64_t ss, int tok) -> const char* {
+    tok = tok > last_rel ? last_rel : tok;
+    const int h = tok >> 4;
+    int pidx, s16;
+    if (hshift >= 0) { pidx = h >> hshift; s16 = h & (hpp - 1); }
+    else { pidx = h / hpp; s16 = h - pidx * hpp; }
+    const int pg = __shfl(pidx < 64 ? pg0 : pg1, pidx & 63);
+    return base + (int64_t)pg * sp + (int64_t)(s16 * 16 + (tok & 15)) * ss;
+  };
+
+  // Q rows as MFMA B operand (lane (g, n): row row0 + n, dims kk*32 + g*8 .. +7)
   vec8 qreg[KK];
-  {
-    const int r = row0 + n;
-    int s = -1;
-    if (r < R) s = qt[r / G];
-    const bool ok = (unsigned)s < (unsigned)p.batch;
-    const T* qrow = (const T*)p.q + (ok ? ((int64_t)s * p.q_stride_b + (int64_t)(head * G + r % G) * p.q_stride_h) : 0);
+  auto load_q = [&]() {
+    const bool ok = (row0 + n < R) && ((unsigned)my_seq_raw < (unsigned)p.batch);
+    const T* qrow = (const T*)p.q + (ok ? ((int64_t)my_seq_raw * p.q_stride_b + (int64_t)my_hq * p.q_stride_h) : 0);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       u32x4 raw = u32x4{0u, 0u, 0u, 0u};
       if (ok) raw = *(const u32x4*)(qrow + kk * 32 + g * 8);
       qreg[kk] = __builtin_bit_cast(vec8, raw);
-    }
-  }
-  __syncthreads();  // s_pages visible
-
-  const int nsteps = (t_end - t_begin + kStepTokens - 1) / kStepTokens;
-  // KV steps of this wave: every 4th one (short boxes) or all of them (tall boxes, where a
-  // wave whose rows are all padding has nothing to do)
-  const int st_first = tall ? ((row0 < R) ? 0 : nsteps) : wave;
-  const int st_stride = tall ? 1 : kWaves;
-  const bool pow2 = (page & (page - 1)) == 0;
-  const int pshift = 31 - __builtin_clz(page);
-  const T* __restrict__ kbase = (const T*)p.k + (int64_t)head * p.k_stride_h;
-  const T* __restrict__ vbase = (const T*)p.v + (int64_t)head * p.v_stride_h;
-
-  // address of token (chunk-relative index rel) in K or V
-  auto token_ptr = [&](const T* base, int64_t stride_page, int64_t stride_slot, int rel) {
-    int pidx, sl;
-    if (pow2) { pidx = rel >> pshift; sl = rel & (page - 1); }
-    else { pidx = rel / page; sl = rel - pidx * page; }
-    return base + (int64_t)s_pages[pidx] * stride_page + (int64_t)sl * stride_slot;
-  };
-  const int last_rel = t_end - t_begin - 1;
-
-  u32x4 kraw[2][KK], vraw[NV];
-  auto load_step = [&](int st) {
-    const int rel0 = st * kStepTokens;
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      int rel = rel0 + a * 16 + n;
-      rel = rel > last_rel ? last_rel : rel;
-      const T* row = token_ptr(kbase, p.k_stride_page, p.k_stride_slot, rel) + g * 8;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kraw[a][kk] = *(const u32x4*)(row + kk * 32);
-    }
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int piece = j * 64 + lane;
-      int rel = rel0 + piece / CPR;
-      rel = rel > last_rel ? last_rel : rel;
-      const T* row = token_ptr(vbase, p.v_stride_page, p.v_stride_slot, rel);
-      vraw[j] = *(const u32x4*)(row + (piece % CPR) * 8);
     }
   };
 
@@ -208,38 +219,17 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
 #pragma unroll
   for (int db = 0; db < DB; ++db) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  char* vstage = smem + wave * VSTAGE;
-  if (st_first < nsteps) load_step(st_first);
-
-  for (int st = st_first; st < nsteps; st += st_stride) {
-    // current tile -> registers of this iteration; start fetching the next one
-    u32x4 kcur[2][KK], vcur[NV];
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = kraw[a][kk];
-#pragma unroll
-    for (int j = 0; j < NV; ++j) vcur[j] = vraw[j];
-    if (st + st_stride < nsteps) load_step(st + st_stride);
-
-    // V tile -> this wave's LDS region, row-major with padded rows
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int piece = j * 64 + lane;
-      *(PAT_LDS u32x4*)((PAT_LDS char*)vstage + (piece / CPR) * RS + (piece % CPR) * 16) = vcur[j];
-    }
-
-    // S^T = K.Q^T for the two 16-token halves of the step
+  // One 32-token step of online-softmax attention for this wave's 16 rows. k_op(a, kk) yields the
+  // K operand of half a / k-step kk; vtile is a row-major V tile in LDS with row stride RSV.
+  auto attend = [&](auto k_op, const PAT_LDS char* vtile, int t0) {
     f32x4 sc[2];
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk)
-        acc = E::mfma(__builtin_bit_cast(vec8, kcur[a][kk]), qreg[kk], acc);
+      for (int kk = 0; kk < KK; ++kk) acc = E::mfma(k_op(a, kk), qreg[kk], acc);
       sc[a] = acc * p.scale_log2;
     }
-    const int t0 = t_begin + st * kStepTokens;
     if (t0 + kStepTokens > t_end) {
 #pragma unroll
       for (int a = 0; a < 2; ++a)
@@ -247,8 +237,7 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
         for (int i = 0; i < 4; ++i)
           if (t0 + a * 16 + g * 4 + i >= t_end) sc[a][i] = neg_inf();
     }
-
-    // online softmax; the row's running max is shared by its 4 lanes, the sum stays per lane
+    // the row's running max is shared by its 4 lanes, the sum stays per lane until the end
     float mx = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
                      fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
     mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -267,73 +256,179 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
         pv[a * 4 + i] = (T)e;
       }
     l_run = l_run * alpha + psum;
-
     // O^T += V^T.P^T. V^T operand: lane (g, n) of d-block db gets 8 tokens of column db*16 + n:
     // tokens g*4..g*4+3 of each 16-token half, matching the accumulator layout of S^T.
-    {
-      const int rrow = g * 4 + (n >> 2);
-      const PAT_LDS char* src = (const PAT_LDS char*)vstage + rrow * RS + (n & 3) * 8;
+    const PAT_LDS char* src = vtile + (g * 4 + (n >> 2)) * RSV + (n & 3) * 8;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + db * 32));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + 16 * RS + db * 32));
-        s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        acc_o[db] = acc_o[db] * alpha;
-        acc_o[db] = E::mfma(__builtin_bit_cast(vec8, both), pv, acc_o[db]);
+    for (int db = 0; db < DB; ++db) {
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + db * 32));
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + 16 * RSV + db * 32));
+      s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      acc_o[db] = acc_o[db] * alpha;
+      acc_o[db] = E::mfma(__builtin_bit_cast(vec8, both), pv, acc_o[db]);
+    }
+  };
+
+  if (shared_tiles) {
+    // =========================== tall box: tiles shared through LDS ===========================
+    // Each step's K and V tile is fetched once per workgroup: thread t loads pieces t, t + 256 ..
+    // of the tile (16 lanes cover one 256-byte row), PF steps ahead, and drops them into one of
+    // two LDS stages; after a barrier every wave runs its own 16 rows against the stage.
+    u32x4 kst[PF][NP], vst[PF][NP];
+    int tok_in[NP];
+    unsigned koff[NP], voff[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      tok_in[i] = (i * kThreads + tid) / CPR;                 // token of the step, 0..31
+      const unsigned col = ((i * kThreads + tid) % CPR) * 16;
+      koff[i] = (unsigned)((tok_in[i] & 15) * kss) + col;
+      voff[i] = (unsigned)((tok_in[i] & 15) * vss) + col;
+    }
+    auto fetch = [&](int st, u32x4 (&kd)[NP], u32x4 (&vd)[NP]) {
+      if ((st + 1) * kStepTokens <= ntok) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const int h = __builtin_amdgcn_readfirstlane(st * 2 + (tok_in[i] >> 4));   // uniform over the wave
+          kd[i] = *(const u32x4*)(half_base(kbase, ksp, kss, h) + koff[i]);
+          vd[i] = *(const u32x4*)(half_base(vbase, vsp, vss, h) + voff[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const unsigned col = ((i * kThreads + tid) % CPR) * 16;
+          kd[i] = *(const u32x4*)(lane_row(kbase, ksp, kss, st * kStepTokens + tok_in[i]) + col);
+          vd[i] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + tok_in[i]) + col);
+        }
+      }
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s)
+      if (s < nsteps) fetch(s, kst[s], vst[s]);
+    load_q();
+#ifdef PAT_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PAT_STAMP(2);
+#endif
+    for (int st0 = 0; st0 < nsteps; st0 += PF) {
+#pragma unroll
+      for (int s = 0; s < PF; ++s) {
+        const int st = st0 + s;
+        if (st >= nsteps) break;
+        PAT_LDS char* stage = (PAT_LDS char*)smem + (st & 1) * SHARED;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const int tok_in = (i * kThreads + tid) / CPR;
+          const int col16 = ((i * kThreads + tid) % CPR) * 16;
+          *(PAT_LDS u32x4*)(stage + tok_in * RSK + col16) = kst[s][i];
+          *(PAT_LDS u32x4*)(stage + kStepTokens * RSK + tok_in * RSV + col16) = vst[s][i];
+        }
+        if (st + PF < nsteps) fetch(st + PF, kst[s], vst[s]);
+        __syncthreads();
+        if (has_rows)
+          attend([&](int a, int kk) { return *(const PAT_LDS vec8*)(stage + (a * 16 + n) * RSK + (kk * 32 + g * 8) * 2); },
+                 stage + kStepTokens * RSK, t_begin + st * kStepTokens);
       }
     }
-  }
-
-  // the row's sum over all of this wave's tokens
-  l_run += __shfl_xor(l_run, 16);
-  l_run += __shfl_xor(l_run, 32);
-
-  if (tall) {
-    // ---- tall box: this wave holds the finished rows row0..row0+15 of the chunk -----------
-    const int r = row0 + n;
-    if (r < R) {
-      const int s = qt[r / G];
-      const int sb = slot_base(r / G);
-      if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
-        const int hq = head * G + r % G;
-        const int64_t prow = ((int64_t)s * p.heads + hq) * p.num_slots + sb + chunk;
-        const float inv = 1.f / l_run;
-        float* dst = p.o_part + prow * D + g * 4;
+    PAT_STAMP(3);
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    if (my_slot0 >= 0) {
+      const int64_t prow = my_slot0 + chunk;
+      const float inv = 1.f / l_run;
+      float* dst = p.o_part + prow * D + g * 4;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
-        if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+      for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
+      if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+    }
+  } else {
+    // ====================== short box: KV steps split over the 4 waves ========================
+    // No register double-buffering: a wave loads a step, waits, computes. Keeping the register
+    // count low enough for 3-4 workgroups per CU puts more bytes in flight than prefetching
+    // would, because other waves' loads overlap this wave's compute.
+    load_q();
+    PAT_LDS char* vstage = (PAT_LDS char*)smem + wave * VSTAGE;
+    const unsigned koff = (unsigned)(n * kss) + g * 16;                          // K: row n of a half, dims g*8..
+    const unsigned voff = (unsigned)((lane / CPR) * vss) + (lane % CPR) * 16;    // V: TPL rows per instruction
+    for (int st = wave; st < nsteps; st += kWaves) {
+      u32x4 kcur[2][KK], vcur[NV];
+#ifdef PAT_TRACE
+      if (p.debug_mode == 2) {
+        for (int j = 0; j < NV; ++j) vcur[j] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, (unsigned)st};
+        for (int a = 0; a < 2; ++a) for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = u32x4{0x3c003c00u, 0x3c003c00u, (unsigned)st, 0x3c003c00u};
+      } else {
+#endif
+      if ((st + 1) * kStepTokens <= ntok) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const char* vb = half_base(vbase, vsp, vss, st * 2 + a) + voff;
+#pragma unroll
+          for (int j = 0; j < NV / 2; ++j) vcur[a * (NV / 2) + j] = *(const u32x4*)(vb + (int64_t)(j * TPL) * vss);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const char* kb = half_base(kbase, ksp, kss, st * 2 + a) + koff;
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = *(const u32x4*)(kb + kk * 64);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+          vcur[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          const char* kr = lane_row(kbase, ksp, kss, st * kStepTokens + a * 16 + n) + g * 16;
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = *(const u32x4*)(kr + kk * 64);
+        }
       }
+#ifdef PAT_TRACE
+      }
+      if (st == wave) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); PAT_STAMP(2); }
+      if (p.debug_mode == 1) {
+        u32x4 x = u32x4{0u, 0u, 0u, 0u};
+        for (int j = 0; j < NV; ++j) x ^= vcur[j];
+        for (int a = 0; a < 2; ++a) for (int kk = 0; kk < KK; ++kk) x ^= kcur[a][kk];
+        acc_o[0] += __builtin_bit_cast(f32x4, x & 0x007fffffu);
+        continue;
+      }
+#endif
+      // V tile -> this wave's LDS region, row-major with padded rows
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+        *(PAT_LDS u32x4*)(vstage + (j * TPL + lane / CPR) * RSV + (lane % CPR) * 16) = vcur[j];
+      attend([&](int a, int kk) { return __builtin_bit_cast(vec8, kcur[a][kk]); }, vstage, t_begin + st * kStepTokens);
     }
-    return;
-  }
+    PAT_STAMP(3);
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
 
-  // ---- short box: combine the 4 waves' states through LDS and write the partial -------------
-  float* cbuf = (float*)smem;
-  const int crow = tid >> 4;                 // row this thread finalises
-  const int ccol = (tid & 15) * (D / 16);    // its first column
-  __syncthreads();  // every wave is done with its V staging region
-  if (g == 0) { s_m[wave][n] = m_run; s_l[wave][n] = l_run; }
+    // combine the 4 waves' states through LDS and write the partial
+    float* cbuf = (float*)smem;
+    const int crow = tid >> 4;                 // row this thread finalises
+    const int ccol = (tid & 15) * (D / 16);    // its first column
+    __syncthreads();  // every wave is done with its V staging region
+    if (g == 0) { s_m[wave][n] = m_run; s_l[wave][n] = l_run; }
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
-    *(f32x4*)(cbuf + (wave * 16 + n) * OROW + db * 16 + g * 4) = acc_o[db];
-  __syncthreads();
+    for (int db = 0; db < DB; ++db)
+      *(f32x4*)(cbuf + (wave * 16 + n) * OROW + db * 16 + g * 4) = acc_o[db];
+    __syncthreads();
 
-  if (crow < R) {
-    float mw[kWaves], mmax = neg_inf();
+    // the slot of row crow sits in lane crow of every wave
+    const int slot_lo = __shfl((int)(my_slot0 & 0xffffffff), crow);
+    const int slot_hi = __shfl((int)(my_slot0 >> 32), crow);
+    const int64_t cslot0 = ((int64_t)slot_hi << 32) | (unsigned)slot_lo;
+    if (cslot0 >= 0) {
+      float mw[kWaves], mmax = neg_inf();
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) { mw[w] = s_m[w][crow]; mmax = fmaxf(mmax, mw[w]); }
-    float wsum = 0.f, wgt[kWaves];
+      for (int w = 0; w < kWaves; ++w) { mw[w] = s_m[w][crow]; mmax = fmaxf(mmax, mw[w]); }
+      float wsum = 0.f, wgt[kWaves];
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      wgt[w] = fast_exp2(mw[w] - mmax);   // a wave without steps has m = -inf -> weight 0
-      wsum += wgt[w] * s_l[w][crow];
-    }
-    const float inv = 1.f / wsum;
-    const int s = qt[crow / G];
-    const int sb = slot_base(crow / G);
-    if ((unsigned)s < (unsigned)p.batch && sb >= 0) {
-      const int hq = head * G + crow % G;
-      const int64_t prow = ((int64_t)s * p.heads + hq) * p.num_slots + sb + chunk;
+      for (int w = 0; w < kWaves; ++w) {
+        wgt[w] = fast_exp2(mw[w] - mmax);   // a wave without steps has m = -inf -> weight 0
+        wsum += wgt[w] * s_l[w][crow];
+      }
+      const float inv = 1.f / wsum;
+      const int64_t prow = cslot0 + chunk;
       float* dst = p.o_part + prow * D + ccol;
 #pragma unroll
       for (int c = 0; c < D / 16; c += 4) {
@@ -347,6 +442,19 @@ __global__ void __launch_bounds__(kThreads) pat_split_kernel(const SplitParams p
         p.lse_part[prow] = (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f;
     }
   }
+#ifdef PAT_TRACE
+  if (p.trace && tid == 0) {
+    PAT_STAMP(4);
+    unsigned hw, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    long long* t = p.trace + (long long)wg * 8;
+    for (int i = 0; i < 5; ++i) t[i] = tr[i];
+    t[5] = ((long long)xcc << 32) | hw;
+    t[6] = nsteps;
+    t[7] = ((long long)bi << 48) | ((long long)box << 24) | chunk;
+  }
+#endif
 }
 
 // Host launcher: picks the instance for (element type, head_dim).
