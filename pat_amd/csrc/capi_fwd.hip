@@ -119,7 +119,8 @@ int check_args(const pat_fwd_args* a) {
 //    so that this work fills the device with about kTargetWgsPerCU workgroups per CU - few
 //    enough that all are resident at once, so every CU has loads in flight from start to end;
 //  * boxes of 17..64 rows walk the chunk step by step with all 4 waves (one row tile each) and
-//    write 16..32 KB of partial output per workgroup: they get a fixed chunk.
+//    write 16..32 KB of partial output per workgroup: their chunk is at least 256 tokens, and
+//    longer when they alone would still fill the device.
 // PAT_CHUNK_TOKENS / PAT_TALL_CHUNK_TOKENS override the two sizes (tuning aid).
 int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   const int page = a->page_size;
@@ -127,15 +128,25 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   auto round_unit = [&](int64_t c) { return std::max<int64_t>(unit, ceil_div64(c, unit) * unit); };
   const int64_t cap = (int64_t)kMaxChunkPages * page / unit * unit;  // page ids of a chunk sit in 2 VGPRs
   if (cap <= 0) return fail(PAT_ERR_INVALID, "page size too large for one workgroup");
-  int64_t work = 0;
-  for (int i = 0; i < a->num_buckets; ++i)
-    if (row_tiles(a->buckets[i].mnw[0]) == 1)
-      work += (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
+  int64_t work = 0, tall_work = 0;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const int64_t w = (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
+    if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w; else tall_work += w;
+  }
   int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
   if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
-  if (chunk <= 0) chunk = std::max<int64_t>(kMinChunk, std::min<int64_t>(kMaxChunk, work / (kTargetWgsPerCU * kNumCUs)));
-  if (tall <= 0) tall = kTallChunk;
+  if (chunk <= 0) {
+    // whole multiples of 128 tokens: the 4 waves of a workgroup get the same number of steps,
+    // and boxes a little longer than the average do not spill a few tokens into a second chunk
+    chunk = ceil_div64(work / (kTargetWgsPerCU * kNumCUs), 128) * 128;
+    chunk = std::max<int64_t>(kMinChunk, std::min<int64_t>(kMaxChunk, chunk));
+  }
+  if (tall <= 0) {
+    // at least kTallChunk; longer when the tall boxes alone would still fill the device
+    tall = ceil_div64(tall_work / (kTargetWgsPerCU * kNumCUs), 128) * 128;
+    tall = std::max<int64_t>(kTallChunk, std::min<int64_t>(kMaxChunk, tall));
+  }
   g->chunk = (int)std::min(round_unit(chunk), cap);
   g->tall_chunk = (int)std::min(round_unit(tall), cap);
   g->chunks_per_rank = 1;
@@ -252,8 +263,6 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
 #ifdef PAT_TRACE
     sp.trace = nullptr;
     if (const char* env = std::getenv("PAT_TRACE_PTR")) sp.trace = reinterpret_cast<long long*>(std::strtoull(env, nullptr, 0));
-    sp.debug_mode = 0;
-    if (const char* env = std::getenv("PAT_DEBUG_MODE")) sp.debug_mode = std::atoi(env);
 #endif
     if (wg > 0) {
       const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, (unsigned)wg, stream, sp);

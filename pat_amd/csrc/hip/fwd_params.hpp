@@ -49,7 +49,6 @@ struct SplitParams {
   int32_t num_buckets;
 #ifdef PAT_TRACE
   long long* trace;         // debug builds only: 8 timestamps/ids per workgroup
-  int debug_mode;           // debug builds only: 1 = loads without compute, 2 = compute without loads
 #endif
   BucketDev bucket[kMaxBuckets];
 };

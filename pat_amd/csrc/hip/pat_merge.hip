@@ -6,10 +6,11 @@
 // out = sum_i e^(LSE_i - LSE) * O_i, cast to the output type; the final LSE is natural
 // log of the scaled-logit sum.
 //
-// One wave64 per (sequence, head): lanes first scan the row's slot LSEs (slots that
-// no workgroup filled hold -inf and get weight 0), then each lane accumulates
-// head_dim/64 columns over the filled slots, so every partial row is read as one
-// contiguous 256- or 512-byte segment.
+// One wave64 per (sequence, head). The row's slot LSEs are read once, up to 4 per lane,
+// and stay in registers (slots no workgroup filled hold -inf and get weight 0); then each
+// lane accumulates head_dim/64 columns over the filled slots, whose rows are fetched in
+// batches of 16 independent loads. The kernel is a chain of three memory round trips
+// (split count, LSEs, partial rows), which is what its run time consists of.
 #include <hip/hip_runtime.h>
 
 #include "fwd_params.hpp"
@@ -18,40 +19,51 @@ namespace pat {
 
 template <typename T, int D>
 __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
-  constexpr int CPL = D / 64;  // columns per lane
+  constexpr int CPL = D / 64;   // columns per lane
+  constexpr int kRegs = 4;      // LSE registers per lane: up to 256 slots stay in registers
+  constexpr int kBatch = 16;    // partial rows fetched together
   const int lane = threadIdx.x & 63;
   const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (pair >= (int64_t)p.batch * p.heads) return;
   const int s = (int)(pair / p.heads);
   const int hq = (int)(pair % p.heads);
+  const float ninf = -__builtin_inff();
 
-  int nsplit = p.num_split_per_seq[s];
-  nsplit = nsplit < 0 ? 0 : (nsplit > p.max_split ? p.max_split : nsplit);
-  const int nslots = nsplit * p.chunks_per_rank;  // slots are rank-major
   const float* __restrict__ lse = p.lse_part + pair * p.num_slots;
   const float* __restrict__ op = p.o_part + pair * (int64_t)p.num_slots * D;
+  int nsplit = p.num_split_per_seq[s];
+  nsplit = nsplit < 0 ? 0 : (nsplit > p.max_split ? p.max_split : nsplit);
+  const int nslots = nsplit * p.chunks_per_rank;  // slots are box-major
 
-  // pass 1: global max and sum of the slot LSEs
-  float mx = -__builtin_inff();
-  for (int i = lane; i < nslots; i += 64) mx = fmaxf(mx, lse[i]);
+  // slot LSEs -> registers (slots past 256 are re-read below; no plan of the default buckets
+  // gets there: 32 splits x 64 chunks would)
+  float mine[kRegs];
+  float mx = ninf;
+#pragma unroll
+  for (int r = 0; r < kRegs; ++r) {
+    const int i = r * 64 + lane;
+    mine[r] = (i < nslots) ? lse[i] : ninf;
+    mx = fmaxf(mx, mine[r]);
+  }
+  for (int i = kRegs * 64 + lane; i < nslots; i += 64) mx = fmaxf(mx, lse[i]);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   float sum = 0.f;
-  if (mx > -__builtin_inff())
-    for (int i = lane; i < nslots; i += 64) sum += __expf(lse[i] - mx);
+  if (mx > ninf) {
+#pragma unroll
+    for (int r = 0; r < kRegs; ++r) sum += __expf(mine[r] - mx);   // exp(-inf) = 0
+    for (int i = kRegs * 64 + lane; i < nslots; i += 64) sum += __expf(lse[i] - mx);
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  const float total = (sum > 0.f) ? mx + logf(sum) : -__builtin_inff();
+  const float total = (sum > 0.f) ? mx + logf(sum) : ninf;
 
-  // pass 2: weighted sum of the filled slots, 8 at a time so that their loads overlap
-  constexpr int kBatch = 8;
   float acc[CPL];
 #pragma unroll
   for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
-  for (int base = 0; base < nslots; base += 64) {
-    const int i = base + lane;
-    const float mine = (i < nslots) ? lse[i] : -__builtin_inff();
-    const float w_mine = (mine > -__builtin_inff()) ? __expf(mine - total) : 0.f;
+
+  // weighted sum of the filled slots of one 64-slot group
+  auto accumulate = [&](int base, float w_mine) {
     unsigned long long live = __ballot(w_mine > 0.f);
     while (live) {
       int js[kBatch];
@@ -83,6 +95,16 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
         }
       }
     }
+  };
+#pragma unroll
+  for (int r = 0; r < kRegs; ++r) {
+    if (r * 64 >= nslots) break;
+    accumulate(r * 64, (mine[r] > ninf) ? __expf(mine[r] - total) : 0.f);
+  }
+  for (int base = kRegs * 64; base < nslots; base += 64) {
+    const int i = base + lane;
+    const float l = (i < nslots) ? lse[i] : ninf;
+    accumulate(base, (l > ninf) ? __expf(l - total) : 0.f);
   }
 
   T* dst = (T*)p.out + (int64_t)s * p.o_stride_b + (int64_t)hq * p.o_stride_h + lane * CPL;

@@ -77,7 +77,8 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
   constexpr int SHARED = kStepTokens * (RSK + RSV);    // one shared K + V stage
   constexpr int OROW = D + 4;            // padded row of the combine buffer, floats
   constexpr int COMBINE = kWaves * 16 * OROW * 4;
-  constexpr int SMEM0 = (kWaves * VSTAGE > COMBINE) ? kWaves * VSTAGE : COMBINE;
+  constexpr int WSTAGE = VSTAGE;                       // one wave's private staging (V only)
+  constexpr int SMEM0 = (kWaves * WSTAGE > COMBINE) ? kWaves * WSTAGE : COMBINE;
   constexpr int SMEM = (SMEM0 > 2 * SHARED) ? SMEM0 : 2 * SHARED;
 
   __shared__ __attribute__((aligned(16))) char smem[SMEM];
@@ -342,21 +343,17 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
     }
   } else {
     // ====================== short box: KV steps split over the 4 waves ========================
-    // No register double-buffering: a wave loads a step, waits, computes. Keeping the register
-    // count low enough for 3-4 workgroups per CU puts more bytes in flight than prefetching
-    // would, because other waves' loads overlap this wave's compute.
+    // No register double-buffering: a wave loads a step, waits, computes; other waves' loads
+    // overlap its compute (2 or 3 resident workgroups per CU measured the same).
     load_q();
-    PAT_LDS char* vstage = (PAT_LDS char*)smem + wave * VSTAGE;
+    // K rows go straight into MFMA operand layout (16 rows x 64 bytes per load instruction); V rows
+    // are fetched TPL whole rows per instruction and staged in this wave's LDS region. (Staging K
+    // the same way and reading operands back from LDS was measured: no faster, twice the LDS.)
+    PAT_LDS char* vstage = (PAT_LDS char*)smem + wave * WSTAGE;
     const unsigned koff = (unsigned)(n * kss) + g * 16;                          // K: row n of a half, dims g*8..
     const unsigned voff = (unsigned)((lane / CPR) * vss) + (lane % CPR) * 16;    // V: TPL rows per instruction
     for (int st = wave; st < nsteps; st += kWaves) {
       u32x4 kcur[2][KK], vcur[NV];
-#ifdef PAT_TRACE
-      if (p.debug_mode == 2) {
-        for (int j = 0; j < NV; ++j) vcur[j] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, (unsigned)st};
-        for (int a = 0; a < 2; ++a) for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = u32x4{0x3c003c00u, 0x3c003c00u, (unsigned)st, 0x3c003c00u};
-      } else {
-#endif
       if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
@@ -382,15 +379,7 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
         }
       }
 #ifdef PAT_TRACE
-      }
       if (st == wave) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); PAT_STAMP(2); }
-      if (p.debug_mode == 1) {
-        u32x4 x = u32x4{0u, 0u, 0u, 0u};
-        for (int j = 0; j < NV; ++j) x ^= vcur[j];
-        for (int a = 0; a < 2; ++a) for (int kk = 0; kk < KK; ++kk) x ^= kcur[a][kk];
-        acc_o[0] += __builtin_bit_cast(f32x4, x & 0x007fffffu);
-        continue;
-      }
 #endif
       // V tile -> this wave's LDS region, row-major with padded rows
 #pragma unroll
@@ -406,7 +395,7 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
     float* cbuf = (float*)smem;
     const int crow = tid >> 4;                 // row this thread finalises
     const int ccol = (tid & 15) * (D / 16);    // its first column
-    __syncthreads();  // every wave is done with its V staging region
+    __syncthreads();  // every wave is done with its staging region
     if (g == 0) { s_m[wave][n] = m_run; s_l[wave][n] = l_run; }
 #pragma unroll
     for (int db = 0; db < DB; ++db)
