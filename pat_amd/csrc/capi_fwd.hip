@@ -15,8 +15,7 @@
 namespace pat {
 
 // defined next to the kernels (hip/pat_split.hip, hip/pat_merge.hip)
-hipError_t launch_split(bool bf16, int head_dim, unsigned workgroups, hipStream_t stream,
-                        const SplitParams& params);
+hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const SplitParams& params);
 hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params);
 
 namespace {
@@ -164,7 +163,8 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     g->total_wgs += (int64_t)a->buckets[i].num_boxes * n * a->kv_heads;
   }
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
-  if (g->total_wgs > INT32_MAX) return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
+  if (g->total_wgs / a->kv_heads > (int64_t)kGridItemsY * 65535)
+    return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   return PAT_OK;
 }
 
@@ -243,11 +243,12 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   // one launch over all buckets, in plan order (tall, long boxes come first in the default order)
   {
     int nb = 0;
-    int64_t wg = 0;
+    int64_t items = 0;
+    for (int i = 0; i < kMaxBuckets; ++i) sp.item_begin[i] = INT32_MAX;
     for (int i = 0; i < args->num_buckets; ++i) {
       const pat_fwd_bucket& b = args->buckets[i];
       if (b.num_boxes == 0) continue;
-      BucketDev& d = sp.bucket[nb++];
+      BucketDev& d = sp.bucket[nb];
       d.q_table = b.q_table; d.block_table = b.block_table; d.num_seqs = b.num_seqs;
       d.rank = b.rank; d.kv = b.kv; d.q_slot = b.q_slot;
       d.q_stride = (int32_t)b.q_table_stride; d.bt_stride = (int32_t)b.block_table_stride;
@@ -255,17 +256,19 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
       d.chunk_tokens = g.bucket_chunk[i];
       d.chunks = g.bucket_chunks[i];
       d.row_tiles = row_tiles(b.mnw[0]);
-      d.wg_begin = (int32_t)wg;
-      wg += (int64_t)b.num_boxes * d.chunks * args->kv_heads;
+      d.item_begin = (int32_t)items;
+      sp.item_begin[nb] = (int32_t)items;
+      ++nb;
+      items += (int64_t)b.num_boxes * d.chunks;
     }
     sp.num_buckets = nb;
-    sp.total_wgs = (int32_t)wg;
+    sp.total_items = (int32_t)items;
 #ifdef PAT_TRACE
     sp.trace = nullptr;
     if (const char* env = std::getenv("PAT_TRACE_PTR")) sp.trace = reinterpret_cast<long long*>(std::strtoull(env, nullptr, 0));
 #endif
-    if (wg > 0) {
-      const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, (unsigned)wg, stream, sp);
+    if (items > 0) {
+      const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, sp);
       if (e != hipSuccess) return hip_fail(e, "split kernel launch");
     }
   }

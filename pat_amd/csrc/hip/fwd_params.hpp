@@ -8,6 +8,7 @@ constexpr int kMaxBuckets = 12;    // the reference dispatches 12 tile shapes (s
 constexpr int kWaves = 4;          // waves per split-kernel workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kStepTokens = 32;    // KV tokens one wave consumes per loop iteration
+constexpr int kGridItemsY = 32768;  // work items per grid.y slice (grid.z counts slices)
 constexpr int kMaxChunkPages = 128; // page ids of a chunk: two per lane of a wave
 
 // One tile bucket as the split kernel sees it.
@@ -25,7 +26,7 @@ struct BucketDev {
   int32_t max_blocks;    // valid block_table columns
   int32_t chunk_tokens;  // KV tokens per workgroup (multiple of 32 and of page_size)
   int32_t chunks;        // workgroups along the KV axis reserved per box
-  int32_t wg_begin;      // first workgroup of this bucket
+  int32_t item_begin;    // first work item (box, chunk) of this bucket
   int32_t row_tiles;     // 16-row tiles per box: 1 = KV steps split over waves, 2/4 = one wave per tile
   int32_t pad_;
 };
@@ -44,9 +45,10 @@ struct SplitParams {
   int32_t chunks_per_rank;  // slots reserved per CTA_rank
   int32_t num_slots;        // max_split_per_seq * chunks_per_rank
   int32_t max_split;
-  int32_t total_wgs;
+  int32_t total_items;      // work items (box, chunk) over all buckets; the grid is (kv_heads, items)
   float scale_log2;         // softmax_scale * log2(e)
   int32_t num_buckets;
+  int32_t item_begin[kMaxBuckets];  // copy of bucket[i].item_begin at fixed offsets (INT32_MAX past the end)
 #ifdef PAT_TRACE
   long long* trace;         // debug builds only: 8 timestamps/ids per workgroup
 #endif

@@ -9,10 +9,10 @@
 // those tokens plus LSE = max + ln(sum) (csrc/softmax.h:169-188).
 //
 // Mapping to the hardware (this kernel's own design):
-//  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each. The kv-head is the
-//    fastest-varying part of the workgroup index: workgroups are dealt to the 8 XCDs
-//    round-robin, so with 8 kv-heads XCD x serves head x and boxes that share KV pages (the
-//    boxes of one prefix node) find them in that XCD's L2.
+//  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each; grid = (kv heads,
+//    items), so the kv-head is the fastest-varying part of the dispatch order: workgroups are
+//    dealt to the 8 XCDs round-robin, so with 8 kv-heads XCD x serves head x and boxes that
+//    share KV pages (the boxes of one prefix node) find them in that XCD's L2.
 //  * boxes of up to 16 rows (one MFMA row tile): each wave owns every 4th 32-token step of
 //    the chunk on wave-private tiles and runs an independent online softmax; the 4 states are
 //    combined through LDS at the end. K rows are the MFMA A operand of S^T = K.Q^T, so a lane
@@ -60,15 +60,25 @@ template <> struct Elem<__bf16> {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 
+// Tuning knobs (measured on MI355X: depth 1 with 3 workgroups per CU and depth 2 with 2 per CU run
+// the same; deeper rings need 1 workgroup per CU and lose more to fewer resident workgroups than
+// they gain).
+#ifndef PAT_DEPTH
+#define PAT_DEPTH 1   // wave-private tiles: steps a wave keeps in flight
+#endif
+#ifndef PAT_OCC
+#define PAT_OCC 3     // resident workgroups per CU the register budget is sized for
+#endif
 template <typename T, int D>
-__global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParams p) {
+__global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   constexpr int KK = D / 32;             // MFMA k-steps across head_dim in S^T = K.Q^T
   constexpr int DB = D / 16;             // 16-wide head_dim blocks of O^T
   constexpr int NV = D / 16;             // 16-byte V loads per lane per step (wave-private tiles)
   constexpr int NP = D / 64;             // 16-byte K (and V) loads per thread per step (shared tiles)
-  constexpr int PF = 2;                  // shared tiles: steps kept in flight per workgroup
+  constexpr int PF = 4;                  // shared tiles: steps kept in flight per workgroup
+  constexpr int DEPTH = PAT_DEPTH;       // wave-private tiles: steps kept in flight per wave
   constexpr int CPR = D / 8;             // 16-byte pieces per token row
   constexpr int TPL = 64 / CPR;          // tokens covered by one wave-wide load instruction
   constexpr int RSK = D * 2 + 16;        // LDS row stride of a K tile (conflict-free 16-byte row reads)
@@ -98,17 +108,22 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
   const int n = lane & 15;   // index inside the group
 
   // ---- which (bucket, box, chunk, kv-head) is this workgroup? ---------------------------
-  const int wg = blockIdx.x;
+  // grid = (kv heads, work items): the head is the fastest-varying part of the dispatch order.
+  // The bucket is found from a table at fixed kernel-argument offsets and its descriptor is
+  // fetched whole, so the decode costs two scalar-memory round trips, not one per field.
+  const int head = blockIdx.x;
+  const int item = blockIdx.z * kGridItemsY + blockIdx.y;   // past the last item: lands past the last box
   int bi = 0;
-  for (int i = 1; i < p.num_buckets; ++i)
-    if (wg >= p.bucket[i].wg_begin) bi = i;
-  const BucketDev& bk = p.bucket[bi];
-  int local = wg - bk.wg_begin;
-  const int head = local % p.kv_heads;
-  local /= p.kv_heads;
+#pragma unroll
+  for (int i = 1; i < kMaxBuckets; ++i) bi += (item >= p.item_begin[i]) ? 1 : 0;
+  const BucketDev bk = p.bucket[bi];
+  const int local = item - bk.item_begin;
   const int chunk = local % bk.chunks;
   const int box = local / bk.chunks;
   if (box >= bk.num_boxes) return;
+#ifdef PAT_TRACE
+  const int wg = item * p.kv_heads + head;
+#endif
 
   // Boxes of up to 16 rows: the 4 waves split the chunk's steps, each on wave-private tiles.
   // Taller boxes: wave w owns rows 16w..16w+15, all waves walk the same steps on tiles shared
@@ -343,8 +358,10 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
     }
   } else {
     // ====================== short box: KV steps split over the 4 waves ========================
-    // No register double-buffering: a wave loads a step, waits, computes; other waves' loads
-    // overlap its compute (2 or 3 resident workgroups per CU measured the same).
+    // Each wave keeps DEPTH of its steps in flight in a ring of register buffers: when a step has
+    // been consumed its buffer is refilled with the step DEPTH rounds ahead. The chunk is short
+    // (a few steps per wave), so most of a workgroup's bytes are requested before the first
+    // arrives: the kernel's run time is then set by bandwidth, not by a chain of round trips.
     load_q();
     // K rows go straight into MFMA operand layout (16 rows x 64 bytes per load instruction); V rows
     // are fetched TPL whole rows per instruction and staged in this wave's LDS region. (Staging K
@@ -352,40 +369,57 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
     PAT_LDS char* vstage = (PAT_LDS char*)smem + wave * WSTAGE;
     const unsigned koff = (unsigned)(n * kss) + g * 16;                          // K: row n of a half, dims g*8..
     const unsigned voff = (unsigned)((lane / CPR) * vss) + (lane % CPR) * 16;    // V: TPL rows per instruction
-    for (int st = wave; st < nsteps; st += kWaves) {
-      u32x4 kcur[2][KK], vcur[NV];
+    u32x4 kring[DEPTH][2][KK], vring[DEPTH][NV];
+    auto fetch = [&](int st, u32x4 (&kd)[2][KK], u32x4 (&vd)[NV]) {
       if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
           const char* vb = half_base(vbase, vsp, vss, st * 2 + a) + voff;
 #pragma unroll
-          for (int j = 0; j < NV / 2; ++j) vcur[a * (NV / 2) + j] = *(const u32x4*)(vb + (int64_t)(j * TPL) * vss);
+          for (int j = 0; j < NV / 2; ++j) vd[a * (NV / 2) + j] = *(const u32x4*)(vb + (int64_t)(j * TPL) * vss);
         }
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
           const char* kb = half_base(kbase, ksp, kss, st * 2 + a) + koff;
 #pragma unroll
-          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = *(const u32x4*)(kb + kk * 64);
+          for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kb + kk * 64);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < NV; ++j)
-          vcur[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
+          vd[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
           const char* kr = lane_row(kbase, ksp, kss, st * kStepTokens + a * 16 + n) + g * 16;
 #pragma unroll
-          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = *(const u32x4*)(kr + kk * 64);
+          for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kr + kk * 64);
         }
       }
-#ifdef PAT_TRACE
-      if (st == wave) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); PAT_STAMP(2); }
-#endif
-      // V tile -> this wave's LDS region, row-major with padded rows
+    };
 #pragma unroll
-      for (int j = 0; j < NV; ++j)
-        *(PAT_LDS u32x4*)(vstage + (j * TPL + lane / CPR) * RSV + (lane % CPR) * 16) = vcur[j];
-      attend([&](int a, int kk) { return __builtin_bit_cast(vec8, kcur[a][kk]); }, vstage, t_begin + st * kStepTokens);
+    for (int d = 0; d < DEPTH; ++d)
+      if (wave + d * kWaves < nsteps) fetch(wave + d * kWaves, kring[d], vring[d]);
+#ifdef PAT_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PAT_STAMP(2);
+#endif
+    for (int st0 = wave; st0 < nsteps; st0 += DEPTH * kWaves) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int st = st0 + d * kWaves;
+        if (st >= nsteps) break;
+        // V tile -> this wave's LDS region, row-major with padded rows
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+          *(PAT_LDS u32x4*)(vstage + (j * TPL + lane / CPR) * RSV + (lane % CPR) * 16) = vring[d][j];
+        u32x4 kcur[2][KK];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = kring[d][a][kk];
+        attend([&](int a, int kk) { return __builtin_bit_cast(vec8, kcur[a][kk]); }, vstage, t_begin + st * kStepTokens);
+        if (st + DEPTH * kWaves < nsteps) fetch(st + DEPTH * kWaves, kring[d], vring[d]);
+      }
     }
     PAT_STAMP(3);
     l_run += __shfl_xor(l_run, 16);
@@ -447,12 +481,14 @@ __global__ void __launch_bounds__(kThreads, 3) pat_split_kernel(const SplitParam
 }
 
 // Host launcher: picks the instance for (element type, head_dim).
-hipError_t launch_split(bool bf16, int head_dim, unsigned workgroups, hipStream_t stream,
-                        const SplitParams& params) {
+hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const SplitParams& params) {
   void (*fn)(const SplitParams);
   if (bf16) fn = head_dim == 64 ? pat_split_kernel<__bf16, 64> : pat_split_kernel<__bf16, 128>;
   else fn = head_dim == 64 ? pat_split_kernel<_Float16, 64> : pat_split_kernel<_Float16, 128>;
-  hipLaunchKernelGGL(fn, dim3(workgroups), dim3(kThreads), 0, stream, params);
+  const unsigned items = (unsigned)params.total_items;
+  const dim3 grid((unsigned)params.kv_heads, items < (unsigned)kGridItemsY ? items : (unsigned)kGridItemsY,
+                  (items + kGridItemsY - 1) / kGridItemsY);
+  hipLaunchKernelGGL(fn, grid, dim3(kThreads), 0, stream, params);
   return hipGetLastError();
 }
 
