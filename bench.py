@@ -30,6 +30,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 INFINITY_CACHE_BYTES = 256 << 20
+# HBM bytes per split-kernel launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by
+# the same counter's reading for a 1 GiB copy kernel (profiles/pat_split_kernel_<workload>.md)
+MEASURED_TRAFFIC_BYTES = {"c2": 99_180_000}
 
 WORKLOAD_TEXT = {
     "c1": "8 req, 256 shared + 32 private tokens, 8/8 heads, d64, fp16",
@@ -77,6 +80,10 @@ def main() -> None:
     ap.add_argument("--no-oblivious", action="store_true")
     ap.add_argument("--kernel-loop-only", action="store_true",
                     help="run only warmup + timed steps (for rocprofv3 runs)")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="instead of the benchmark, run a plain elementwise copy of this many MiB 5 times "
+                         "(reads N, writes N bytes): the known-size kernel that scales rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path has no cross-GPU step); use --gpus 1",
@@ -89,6 +96,15 @@ def main() -> None:
     assert torch.cuda.is_available(), "bench.py needs an AMD GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.calibrate_copy_mib > 0:
+        n = a.calibrate_copy_mib << 20
+        src = torch.ones(n // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)        # one elementwise kernel: reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_copy_bytes": n, "launches": 5}))
+        return
     lib = _lib.load()
     hip = Hip()
 
@@ -205,11 +221,8 @@ def main() -> None:
                      "traffic": None},
     }
 
-    # measured HBM traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE), if recorded
-    traffic_file = os.path.join(ROOT, "profiles", f"traffic_{a.workload}.json")
-    if os.path.exists(traffic_file):
-        with open(traffic_file) as f:
-            result["roofline"]["traffic"] = json.load(f).get("bytes_per_launch")
+    if a.seed == 0:
+        result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.workload)
 
     if not a.no_oblivious:
         ob = workloads.oblivious_plan(w, dev)
