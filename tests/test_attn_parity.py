@@ -142,6 +142,44 @@ def test_ragged_random_forest(dtype, d, heads):
     _assert_close("forest", out, lse, ref_out, ref_lse, dtype)
 
 
+@pytest.mark.parametrize("heads,k", [((8, 8), 64), ((32, 8), 16), ((16, 4), 5)])
+def test_legacy_flat_schedule_plan(heads, k):
+    # the v0 entry `schedule`: plans in lexsort order; q goes in sorted, the output comes back through
+    # reverse_index (the reordering the reference's vLLM v0 backend did around the kernel)
+    print(f"[case] legacy schedule() plan heads={heads} k={k}", flush=True)
+    import random
+    from pat_amd import schedule
+    dev = _device()
+    r = random.Random(k)
+    rows, lens, nxt = [], [], 0
+    for _ in range(45):
+        row = []
+        if rows and r.random() < 0.85:
+            base = rows[r.randrange(len(rows))]
+            row = list(base[:r.randint(0, len(base) - 1)])
+        extra = r.randint(1, 24)
+        row += list(range(nxt, nxt + extra)); nxt += extra
+        rows.append(row)
+        lens.append(len(row) * 16 - r.randint(0, 15))
+    perm = list(range(1, nxt + 1)); r.shuffle(perm)          # page 0 is the table's padding value
+    rows = [[perm[x] for x in row] for row in rows]
+    w = workloads.Workload("flat", heads[0], heads[1], 128, torch.float16, 16, lens, rows, nxt + 1, 0, 5)
+    q, k_cache, v_cache = w.tensors(dev)
+    ki = schedule(lens, rows, 16, k, None, heads[0] // heads[1])
+    ki.to_tensor(device=dev)
+    order = ki.sort_index.long()
+    out_sorted = torch.full_like(q, float("nan"))
+    lse_sorted = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q[order].contiguous(), k_cache, v_cache, ki.num_split_per_seq, ki.q_tables,
+                             ki.block_tables, ki.num_seqs_per_CTAs, ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs,
+                             ki.max_split_per_seq, ki.max_seqs_in_CTA, ki.max_blocks_in_CTA,
+                             1.0 / math.sqrt(w.head_dim), out_sorted, None, softmax_lse=lse_sorted)
+    torch.cuda.synchronize()
+    back = ki.reverse_index.long()
+    ref_out, ref_lse = _oracle(w, q, k_cache, v_cache)
+    _assert_close("legacy schedule", out_sorted[back], lse_sorted[back], ref_out, ref_lse, torch.float16)
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
