@@ -165,6 +165,9 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
   if (g->total_wgs / a->kv_heads > (int64_t)kGridItemsY * 65535)
     return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
+  // the kernels index partial rows with 32-bit integers
+  if ((int64_t)a->batch * a->heads * g->num_slots >= ((int64_t)1 << 31))
+    return fail(PAT_ERR_INVALID, "batch * heads * partial slots must stay below 2^31");
   return PAT_OK;
 }
 

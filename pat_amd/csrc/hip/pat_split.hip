@@ -31,6 +31,7 @@
 #include <hip/hip_runtime.h>
 
 #include "fwd_params.hpp"
+#include "lane_ops.hpp"
 
 namespace pat {
 
@@ -168,8 +169,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
                       ((unsigned)my_ord < (unsigned)p.max_split);
   const int my_hq = head * G + (row0 + n) % G;
   // first partial slot of (my row, this box); -1: the row is not to be written
-  const int64_t my_slot0 = row_ok ? ((int64_t)my_seq_raw * p.heads + my_hq) * p.num_slots +
-                                        (int64_t)my_ord * p.chunks_per_rank : -1;
+  const int my_slot0 = row_ok ? (my_seq_raw * p.heads + my_hq) * p.num_slots + my_ord * p.chunks_per_rank : -1;
 
   // ---- slots of this box that no workgroup will fill are marked empty (-inf) ------------
   {
@@ -237,7 +237,9 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
 
   // One 32-token step of online-softmax attention for this wave's 16 rows. k_op(a, kk) yields the
   // K operand of half a / k-step kk; vtile is a row-major V tile in LDS with row stride RSV.
-  auto attend = [&](auto k_op, const PAT_LDS char* vtile, int t0) {
+  // after_scores() runs once the K operands have been consumed: the caller refills their
+  // registers there, so the next step's K is in flight during the softmax and the PV product.
+  auto attend = [&](auto k_op, const PAT_LDS char* vtile, int t0, auto after_scores) {
     f32x4 sc[2];
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
@@ -246,6 +248,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       for (int kk = 0; kk < KK; ++kk) acc = E::mfma(k_op(a, kk), qreg[kk], acc);
       sc[a] = acc * p.scale_log2;
     }
+    after_scores();
     if (t0 + kStepTokens > t_end) {
 #pragma unroll
       for (int a = 0; a < 2; ++a)
@@ -256,10 +259,11 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     // the row's running max is shared by its 4 lanes, the sum stays per lane until the end
     float mx = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
                      fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = max_xor32(max_xor16(mx));
     const float m_new = fmaxf(m_run, mx);
     const float alpha = fast_exp2(m_run - m_new);
+    // once the running maxima have settled no row of the wave needs its accumulator rescaled
+    const bool rescale = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;
     m_run = m_new;
     float psum = 0.f;
     vec8 pv;
@@ -280,7 +284,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + db * 32));
       s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + 16 * RSV + db * 32));
       s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      acc_o[db] = acc_o[db] * alpha;
+      if (rescale) acc_o[db] = acc_o[db] * alpha;
       acc_o[db] = E::mfma(__builtin_bit_cast(vec8, both), pv, acc_o[db]);
     }
   };
@@ -342,14 +346,13 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         __syncthreads();
         if (has_rows)
           attend([&](int a, int kk) { return *(const PAT_LDS vec8*)(stage + (a * 16 + n) * RSK + (kk * 32 + g * 8) * 2); },
-                 stage + kStepTokens * RSK, t_begin + st * kStepTokens);
+                 stage + kStepTokens * RSK, t_begin + st * kStepTokens, []() {});
       }
     }
     PAT_STAMP(3);
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
+    l_run = sum_xor32(sum_xor16(l_run));
     if (my_slot0 >= 0) {
-      const int64_t prow = my_slot0 + chunk;
+      const int64_t prow = (int64_t)my_slot0 + chunk;
       const float inv = 1.f / l_run;
       float* dst = p.o_part + prow * D + g * 4;
 #pragma unroll
@@ -370,7 +373,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     const unsigned koff = (unsigned)(n * kss) + g * 16;                          // K: row n of a half, dims g*8..
     const unsigned voff = (unsigned)((lane / CPR) * vss) + (lane % CPR) * 16;    // V: TPL rows per instruction
     u32x4 kring[DEPTH][2][KK], vring[DEPTH][NV];
-    auto fetch = [&](int st, u32x4 (&kd)[2][KK], u32x4 (&vd)[NV]) {
+    auto fetch_v = [&](int st, u32x4 (&vd)[NV]) {
       if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
@@ -378,6 +381,14 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
 #pragma unroll
           for (int j = 0; j < NV / 2; ++j) vd[a * (NV / 2) + j] = *(const u32x4*)(vb + (int64_t)(j * TPL) * vss);
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+          vd[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
+      }
+    };
+    auto fetch_k = [&](int st, u32x4 (&kd)[2][KK]) {
+      if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
           const char* kb = half_base(kbase, ksp, kss, st * 2 + a) + koff;
@@ -385,9 +396,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
           for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kb + kk * 64);
         }
       } else {
-#pragma unroll
-        for (int j = 0; j < NV; ++j)
-          vd[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
           const char* kr = lane_row(kbase, ksp, kss, st * kStepTokens + a * 16 + n) + g * 16;
@@ -398,7 +406,10 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     };
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
-      if (wave + d * kWaves < nsteps) fetch(wave + d * kWaves, kring[d], vring[d]);
+      if (wave + d * kWaves < nsteps) {
+        fetch_v(wave + d * kWaves, vring[d]);
+        fetch_k(wave + d * kWaves, kring[d]);
+      }
 #ifdef PAT_TRACE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     PAT_STAMP(2);
@@ -408,22 +419,21 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       for (int d = 0; d < DEPTH; ++d) {
         const int st = st0 + d * kWaves;
         if (st >= nsteps) break;
-        // V tile -> this wave's LDS region, row-major with padded rows
+        const int nxt = st + DEPTH * kWaves;
+        const bool more = nxt < nsteps;
+        // V tile -> this wave's LDS region, row-major with padded rows; its registers are free
+        // again at once and take the ring's next V tile
 #pragma unroll
         for (int j = 0; j < NV; ++j)
           *(PAT_LDS u32x4*)(vstage + (j * TPL + lane / CPR) * RSV + (lane % CPR) * 16) = vring[d][j];
-        u32x4 kcur[2][KK];
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int kk = 0; kk < KK; ++kk) kcur[a][kk] = kring[d][a][kk];
-        attend([&](int a, int kk) { return __builtin_bit_cast(vec8, kcur[a][kk]); }, vstage, t_begin + st * kStepTokens);
-        if (st + DEPTH * kWaves < nsteps) fetch(st + DEPTH * kWaves, kring[d], vring[d]);
+        if (more) fetch_v(nxt, vring[d]);
+        // the K registers are refilled as soon as the score MFMAs have read them
+        attend([&](int a, int kk) { return __builtin_bit_cast(vec8, kring[d][a][kk]); }, vstage,
+               t_begin + st * kStepTokens, [&]() { if (more) fetch_k(nxt, kring[d]); });
       }
     }
     PAT_STAMP(3);
-    l_run += __shfl_xor(l_run, 16);
-    l_run += __shfl_xor(l_run, 32);
+    l_run = sum_xor32(sum_xor16(l_run));
 
     // combine the 4 waves' states through LDS and write the partial
     float* cbuf = (float*)smem;
@@ -437,9 +447,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     __syncthreads();
 
     // the slot of row crow sits in lane crow of every wave
-    const int slot_lo = __shfl((int)(my_slot0 & 0xffffffff), crow);
-    const int slot_hi = __shfl((int)(my_slot0 >> 32), crow);
-    const int64_t cslot0 = ((int64_t)slot_hi << 32) | (unsigned)slot_lo;
+    const int cslot0 = __shfl(my_slot0, crow);
     if (cslot0 >= 0) {
       float mw[kWaves], mmax = neg_inf();
 #pragma unroll
@@ -451,7 +459,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         wsum += wgt[w] * s_l[w][crow];
       }
       const float inv = 1.f / wsum;
-      const int64_t prow = cslot0 + chunk;
+      const int64_t prow = (int64_t)cslot0 + chunk;
       float* dst = p.o_part + prow * D + ccol;
 #pragma unroll
       for (int c = 0; c < D / 16; c += 4) {
