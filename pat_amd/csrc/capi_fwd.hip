@@ -240,6 +240,10 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   sp.group = args->heads / args->kv_heads;
   sp.page_size = args->page_size; sp.num_pages = args->num_pages;
   sp.chunks_per_rank = g.chunks_per_rank; sp.num_slots = g.num_slots;
+  {
+    const uint64_t hpp = (uint64_t)args->page_size / 16;
+    sp.hpp_magic = hpp > 1 ? (uint32_t)((((uint64_t)1 << 32) + hpp - 1) / hpp) : 0u;
+  }
   sp.max_split = args->max_split_per_seq;
   sp.scale_log2 = args->softmax_scale * 1.4426950408889634f;
 

@@ -48,6 +48,7 @@ struct SplitParams {
   int32_t total_items;      // work items (box, chunk) over all buckets; the grid is (kv_heads, items)
   float scale_log2;         // softmax_scale * log2(e)
   int32_t num_buckets;
+  uint32_t hpp_magic;       // ceil(2^32 / (page_size / 16)): h / (page_size / 16) == umulhi(h, hpp_magic) for h < 2^16; unused when page_size / 16 is a power of two
   int32_t item_begin[kMaxBuckets];  // copy of bucket[i].item_begin at fixed offsets (INT32_MAX past the end)
 #ifdef PAT_TRACE
   long long* trace;         // debug builds only: 8 timestamps/ids per workgroup

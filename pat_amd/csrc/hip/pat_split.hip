@@ -196,11 +196,11 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const char* __restrict__ vbase = (const char*)p.v + (int64_t)head * p.v_stride_h * (int64_t)sizeof(T);
   const int ntok = t_end - t_begin;
 
-  // base address of half h (chunk-relative, uniform, h*16 < ntok)
+  // base address of half h (chunk-relative, uniform, h * 16 <= last_rel)
   auto half_base = [&](const char* base, int64_t sp, int64_t ss, int h) -> const char* {
     int pidx, s16;
     if (hshift >= 0) { pidx = h >> hshift; s16 = h & (hpp - 1); }
-    else { pidx = h / hpp; s16 = h - pidx * hpp; }
+    else { pidx = (int)__umulhi((unsigned)h, p.hpp_magic); s16 = h - pidx * hpp; }
     const int pg = __builtin_amdgcn_readlane(pidx < 64 ? pg0 : pg1, pidx & 63);
     return base + (int64_t)pg * sp + (int64_t)(s16 * 16) * ss;
   };
@@ -212,9 +212,19 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     const int h = tok >> 4;
     int pidx, s16;
     if (hshift >= 0) { pidx = h >> hshift; s16 = h & (hpp - 1); }
-    else { pidx = h / hpp; s16 = h - pidx * hpp; }
+    else { pidx = (int)__umulhi((unsigned)h, p.hpp_magic); s16 = h - pidx * hpp; }
     const int pg = __shfl(pidx < 64 ? pg0 : pg1, pidx & 63);
     return base + (int64_t)pg * sp + (int64_t)(s16 * 16 + (tok & 15)) * ss;
+  };
+
+  // Half h of the chunk as the loads see it (uniform over the wave): the half that holds its rows
+  // and, in `lim`, the last row of that half that exists. Rows past the end of the chunk re-read
+  // the chunk's last token (their scores are masked and their probabilities are 0); a half that
+  // lies wholly past the end stands in for the half of that token.
+  auto half_geom = [&](int h, int& lim) -> int {
+    const int left = last_rel - h * 16;
+    lim = left < 0 ? (last_rel & 15) : (left > 15 ? 15 : left);
+    return left < 0 ? (last_rel >> 4) : h;
   };
 
   // Q rows as MFMA B operand (lane (g, n): row row0 + n, dims kk*32 + g*8 .. +7)
@@ -374,34 +384,29 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     const unsigned voff = (unsigned)((lane / CPR) * vss) + (lane % CPR) * 16;    // V: TPL rows per instruction
     u32x4 kring[DEPTH][2][KK], vring[DEPTH][NV];
     auto fetch_v = [&](int st, u32x4 (&vd)[NV]) {
-      if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const char* vb = half_base(vbase, vsp, vss, st * 2 + a) + voff;
+      for (int a = 0; a < 2; ++a) {
+        int lim;
+        const int h = half_geom(__builtin_amdgcn_readfirstlane(st * 2 + a), lim);
+        const char* vb = half_base(vbase, vsp, vss, h);
 #pragma unroll
-          for (int j = 0; j < NV / 2; ++j) vd[a * (NV / 2) + j] = *(const u32x4*)(vb + (int64_t)(j * TPL) * vss);
+        for (int j = 0; j < NV / 2; ++j) {
+          unsigned vo = voff + (unsigned)(j * TPL) * (unsigned)vss;
+          if (lim < 15 && j * TPL + lane / CPR > lim) vo = (unsigned)(lim * vss) + (lane % CPR) * 16;
+          vd[a * (NV / 2) + j] = *(const u32x4*)(vb + vo);
         }
-      } else {
-#pragma unroll
-        for (int j = 0; j < NV; ++j)
-          vd[j] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + j * TPL + lane / CPR) + (lane % CPR) * 16);
       }
     };
     auto fetch_k = [&](int st, u32x4 (&kd)[2][KK]) {
-      if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const char* kb = half_base(kbase, ksp, kss, st * 2 + a) + koff;
+      for (int a = 0; a < 2; ++a) {
+        int lim;
+        const int h = half_geom(__builtin_amdgcn_readfirstlane(st * 2 + a), lim);
+        const char* kb = half_base(kbase, ksp, kss, h);
+        unsigned ko = koff;
+        if (lim < 15 && n > lim) ko = (unsigned)(lim * kss) + g * 16;
 #pragma unroll
-          for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kb + kk * 64);
-        }
-      } else {
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const char* kr = lane_row(kbase, ksp, kss, st * kStepTokens + a * 16 + n) + g * 16;
-#pragma unroll
-          for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kr + kk * 64);
-        }
+        for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kb + ko + kk * 64);
       }
     };
 #pragma unroll

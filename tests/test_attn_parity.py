@@ -180,6 +180,43 @@ def test_legacy_flat_schedule_plan(heads, k):
     _assert_close("legacy schedule", out_sorted[back], lse_sorted[back], ref_out, ref_lse, torch.float16)
 
 
+@pytest.mark.parametrize("page,dtype,heads", [(48, torch.float16, (32, 8)), (64, torch.bfloat16, (32, 8)),
+                                              (80, torch.float16, (16, 16)), (128, torch.bfloat16, (64, 8)),
+                                              (16, torch.float16, (16, 2))])
+def test_page_sizes_and_tiny_boxes(page, dtype, heads):
+    # pages that are no power of two (the half -> page map divides by a reciprocal), shared nodes whose
+    # length is no multiple of 32 (partial last step of a tall box), requests shorter than one MFMA tile
+    print(f"[case] page {page} {dtype} heads={heads}", flush=True)
+    import random
+    dev = _device()
+    r = random.Random(page)
+    next_block = [0]
+
+    def blocks(n):
+        out = list(range(next_block[0], next_block[0] + n)); next_block[0] += n
+        return out
+
+    rows, lens = [], []
+    root = blocks(3)                                   # 3 pages shared by everybody below
+    for _ in range(20):
+        mid = root + blocks(r.choice([1, 2, 5]))       # shared by 1..4 requests
+        for _ in range(r.randint(1, 4)):
+            own = r.randint(1, 3)
+            row = mid + blocks(own)
+            rows.append(row)
+            lens.append((len(row) - 1) * page + r.randint(1, page))
+    for n in (1, 2, 7, 15, 16, 17, 31, 33):            # tiny private requests
+        rows.append(blocks(-(-n // page)))
+        lens.append(n)
+    perm = list(range(next_block[0])); r.shuffle(perm)
+    rows = [[perm[x] for x in row] for row in rows]
+    w = workloads.Workload("pages", heads[0], heads[1], 128, dtype, page, lens, rows, next_block[0], 0, page)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"page {page}", out, lse, ref_out, ref_lse, dtype)
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
