@@ -286,6 +286,11 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         pv[a * 4 + i] = (T)e;
       }
     l_run = l_run * alpha + psum;
+    if (rescale) {
+      asm volatile("" ::: "memory");   // a real branch: if-converted, the skipped multiplies come back as selects
+#pragma unroll
+      for (int db = 0; db < DB; ++db) acc_o[db] = acc_o[db] * alpha;
+    }
     // O^T += V^T.P^T. V^T operand: lane (g, n) of d-block db gets 8 tokens of column db*16 + n:
     // tokens g*4..g*4+3 of each 16-token half, matching the accumulator layout of S^T.
     const PAT_LDS char* src = vtile + (g * 4 + (n >> 2)) * RSV + (n & 3) * 8;
@@ -294,7 +299,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + db * 32));
       s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PAT_LDS s16x4*)(src + 16 * RSV + db * 32));
       s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      if (rescale) acc_o[db] = acc_o[db] * alpha;
       acc_o[db] = E::mfma(__builtin_bit_cast(vec8, both), pv, acc_o[db]);
     }
   };
