@@ -1,0 +1,153 @@
+"""Decode branch of the vLLM `PREFIX_ATTN` backend, without vLLM.
+
+What plugin/vllm/attention/backends/prefix_attn.py of the flashserve/PAT tree does for the decode
+tokens of a step, as two plain objects a backend (or a test with a stand-in for vLLM's
+AttentionMetadata) can drive:
+
+* `DecodePlan.from_metadata(meta)` is the `decode_metadata` property (:313-338): it drops the
+  prefill rows of the step and starts an `AsyncTree` over the decode requests' lengths and the CPU
+  copy of their block table, so the plan is built while the step's earlier work runs;
+* `decode_attention(...)` is the tail of `PrefixAttentionImpl.forward` (:901-915): it splits
+  vLLM's `[2, num_blocks, block_size, kv_heads, head_size]` cache, waits for the plan and calls
+  `prefix_attn_with_kvcache` on `[B, 1, N, d]` views of the query and output.
+
+* `DecodePlan.advance_step(block_tables_cpu)` is what multi-step decoding needs on top of the
+  reference's `advance_step` (:377-448), which moves the lengths forward but leaves the tree as it
+  was: every request grew by one token, so the work item that holds its tail gets one more token
+  (and, at a page boundary, the next block id) in place on the device; the plan is rebuilt only
+  when that is not possible (a tail shared by several requests, a block row that is full).
+
+`meta` only needs the attributes read here (`num_prefills`, `num_decode_tokens`, `seq_lens`,
+`block_tables`, `block_tables_cpu`, `block_size`, `nheads`, `nheads_kv`,
+`max_decode_query_len`); vLLM's own metadata class has them after the reference's overlay.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, List, Optional, Union
+
+import numpy as np
+import torch
+
+from ._prefix_attn import PrefixTreeCPP, prefix_attn_with_kvcache
+from .async_tree import AsyncTree
+
+__all__ = ["DecodePlan", "decode_attention"]
+
+
+@dataclass
+class DecodePlan:
+    """Per-step decode state shared by all attention layers of the step."""
+    num_decode_tokens: int
+    seq_lens: List[int]
+    block_tables: Optional[torch.Tensor]       # device table of the decode requests
+    tree: Union[AsyncTree, PrefixTreeCPP]
+    max_decode_query_len: int = 1
+    block_size: int = 16
+    nheads: int = 1
+    nheads_kv: int = 1
+    replans: int = 0                           # times advance_step had to plan afresh
+    _tails: Any = None                         # per request (bucket, box) of the item holding its tail
+    _tail_kv: Any = None
+
+    @classmethod
+    def from_metadata(cls, meta: Any) -> Optional["DecodePlan"]:
+        if meta.num_decode_tokens == 0:
+            return None
+        first = meta.num_prefills
+        seq_lens = list(meta.seq_lens[first:])
+        tables = None if meta.block_tables is None else meta.block_tables[first:]
+        table_cpu = meta.block_tables_cpu[first:] if meta.block_tables_cpu.shape[0] != len(seq_lens) \
+            else meta.block_tables_cpu
+        device = tables.device if tables is not None else torch.device("cuda")
+        tree = AsyncTree(block_size=meta.block_size, seq_lens=seq_lens, table=table_cpu, MNWs=None,
+                         HRatio=meta.nheads // meta.nheads_kv, kvHead=meta.nheads_kv, device=device)
+        return cls(num_decode_tokens=meta.num_decode_tokens, seq_lens=seq_lens, block_tables=tables, tree=tree,
+                   max_decode_query_len=getattr(meta, "max_decode_query_len", 1), block_size=meta.block_size,
+                   nheads=meta.nheads, nheads_kv=meta.nheads_kv)
+
+    # ---- multi-step decoding ---------------------------------------------------------------
+    def _ready_tree(self) -> PrefixTreeCPP:
+        return self.tree.tree if isinstance(self.tree, AsyncTree) else self.tree
+
+    def _find_tails(self, table_cpu: torch.Tensor):
+        """For every request the (bucket, box) of the single-request item that ends with the
+        request's last block, or -1 where the tail sits in an item shared with other requests."""
+        info = self._ready_tree().kernel_info
+        bs = self.block_size
+        n = len(self.seq_lens)
+        last_block = np.array([int(table_cpu[i, (self.seq_lens[i] - 1) // bs]) for i in range(n)])
+        tails = np.full((n, 2), -1, dtype=np.int64)
+        self._tail_kv = np.zeros(n, dtype=np.int64)      # host mirror of the tail items' token counts
+        for b in range(len(info.MNWs)):
+            nseq = info.num_seqs_per_CTAs[b].cpu().numpy()
+            kv = info.kv_in_CTAs[b].cpu().numpy()
+            qt = info.q_tables[b].cpu().numpy()
+            bt = info.block_tables[b].cpu().numpy()
+            for box in np.nonzero(nseq == 1)[0]:
+                s = int(qt[box, 0])
+                if kv[box] > 0 and bt[box, (kv[box] - 1) // bs] == last_block[s]:
+                    tails[s] = (b, box)
+                    self._tail_kv[s] = kv[box]
+        return tails
+
+    def _replan(self, table_cpu: torch.Tensor) -> None:
+        device = self._ready_tree().kernel_info.num_split_per_seq.device
+        self.tree = AsyncTree(block_size=self.block_size, seq_lens=list(self.seq_lens), table=table_cpu, MNWs=None,
+                              HRatio=self.nheads // self.nheads_kv, kvHead=self.nheads_kv, device=device)
+        self._tails = None
+        self.replans += 1
+
+    def advance_step(self, block_tables_cpu: torch.Tensor) -> bool:
+        """Every decode request has grown by one token (`block_tables_cpu` already names the block
+        that token went to). Returns True when the plan was updated in place, False when it was
+        rebuilt."""
+        bs = self.block_size
+        table_cpu = block_tables_cpu[-len(self.seq_lens):] if block_tables_cpu.shape[0] != len(self.seq_lens) \
+            else block_tables_cpu
+        if self._tails is None:
+            self._tails = self._find_tails(table_cpu)
+        info = self._ready_tree().kernel_info
+        old = list(self.seq_lens)
+        self.seq_lens = [x + 1 for x in old]
+        if (self._tails[:, 0] < 0).any():
+            self._replan(table_cpu)
+            return False
+        new_blocks = {}                       # bucket -> ([flat positions], [block ids])
+        for s, n_old in enumerate(old):
+            if n_old % bs:
+                continue
+            b, box = self._tails[s]
+            width = info.block_tables[b].shape[1]
+            pos = -(-int(self._tail_kv[s]) // bs)           # blocks the item holds now
+            if pos >= width:
+                self._replan(table_cpu)
+                return False
+            where, ids = new_blocks.setdefault(int(b), ([], []))
+            where.append(int(box) * width + pos)
+            ids.append(int(table_cpu[s, n_old // bs]))
+        self._tail_kv += 1
+        device = info.num_split_per_seq.device
+        for b in range(len(info.MNWs)):
+            boxes = self._tails[self._tails[:, 0] == b, 1]
+            if len(boxes):
+                info.kv_in_CTAs[b].index_add_(0, torch.as_tensor(boxes, device=device),
+                                              torch.ones(len(boxes), dtype=torch.int32, device=device))
+            if b in new_blocks:
+                where, ids = new_blocks[b]
+                info.block_tables[b].view(-1).index_copy_(0, torch.as_tensor(where, device=device),
+                                                          torch.as_tensor(ids, dtype=torch.int32, device=device))
+        return True
+
+
+def decode_attention(decode_query: torch.Tensor, kv_cache: torch.Tensor, plan: DecodePlan, softmax_scale: float,
+                     decode_output: torch.Tensor) -> torch.Tensor:
+    """decode_query / decode_output: [num_decode_tokens, num_heads, head_size];
+    kv_cache: [2, num_blocks, block_size, num_kv_heads, head_size]. Writes and returns decode_output."""
+    assert plan.max_decode_query_len <= 1, \
+        "Speculative decoding with variable length queries is not supported yet."
+    key_cache, value_cache = kv_cache[0], kv_cache[1]
+    tree = plan.tree.tree if isinstance(plan.tree, AsyncTree) else plan.tree
+    prefix_attn_with_kvcache(q=decode_query.unsqueeze(1), k_cache_paged=key_cache, v_cache_paged=value_cache,
+                             tree=tree, softmax_scale=softmax_scale, out=decode_output.unsqueeze(1))
+    return decode_output

@@ -1,0 +1,157 @@
+"""Decode branch of the vLLM backend (pat_amd/vllm_decode.py) driven by a stand-in for vLLM's
+AttentionMetadata: plan construction on the CPU, attention through vLLM's cache layout on the GPU."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from oracle import attn_oracle as ao
+from pat_amd import PrefixTree, workloads
+from pat_amd.vllm_decode import DecodePlan, decode_attention
+from conftest import plan_fields
+
+
+def fake_metadata(w, device, num_prefills=0):
+    """What the backend's metadata holds for a step with `num_prefills` prompt rows ahead of the
+    decode requests of workload w."""
+    pad = torch.zeros(num_prefills, w.padded_table().shape[1], dtype=torch.int32)
+    table_cpu = torch.cat([pad, w.padded_table()])
+    return SimpleNamespace(num_prefills=num_prefills, num_decode_tokens=w.batch,
+                           seq_lens=[7] * num_prefills + list(w.seq_lens),
+                           block_tables=table_cpu.to(device), block_tables_cpu=table_cpu,
+                           block_size=w.page_size, nheads=w.heads, nheads_kv=w.kv_heads, max_decode_query_len=1)
+
+
+def test_decode_plan_drops_prefill_rows_and_matches_scheduler():
+    w = workloads.make("c1", seed=3)
+    plan = DecodePlan.from_metadata(fake_metadata(w, torch.device("cpu"), num_prefills=2))
+    assert plan.num_decode_tokens == w.batch and plan.seq_lens == list(w.seq_lens)
+    assert plan.block_tables.shape[0] == w.batch
+    ref = PrefixTree(w.page_size)
+    ref.build_radix_tree(w.seq_lens, w.rows)
+    want = plan_fields(ref.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads))
+    got = plan.tree.tree.kernel_info
+    assert [list(m) for m in got.MNWs] == want["MNWs"]
+    assert got.num_split_per_seq.tolist() == want["num_split_per_seq"]
+    assert [t.tolist() for t in got.kv_in_CTAs] == want["kv_in_CTAs"]
+
+
+def test_no_decode_tokens_no_plan():
+    meta = SimpleNamespace(num_decode_tokens=0)
+    assert DecodePlan.from_metadata(meta) is None
+
+
+def test_variable_length_decode_queries_are_refused():
+    w = workloads.make("c1", seed=3)
+    plan = DecodePlan.from_metadata(fake_metadata(w, torch.device("cpu")))
+    plan.max_decode_query_len = 2
+    with pytest.raises(AssertionError, match="Speculative decoding"):
+        decode_attention(torch.zeros(w.batch, w.heads, w.head_dim), torch.zeros(2, 1, 16, w.kv_heads, w.head_dim),
+                         plan, 1.0, torch.zeros(w.batch, w.heads, w.head_dim))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["c1", "c2"])
+def test_decode_attention_through_vllm_cache_layout(name):
+    print(f"[case] vLLM decode branch {name}", flush=True)
+    dev = torch.device("cuda:0")
+    w = workloads.make(name, seed=4)
+    q, k, v = w.tensors(dev)
+    kv_cache = torch.stack([k, v])                       # [2, blocks, page, h_kv, d]
+    plan = DecodePlan.from_metadata(fake_metadata(w, dev, num_prefills=1))
+    query = q.squeeze(1).contiguous()                    # [B, N, d]
+    output = torch.full_like(query, float("nan"))
+    for _ in range(2):                                   # every layer of a step reuses the plan
+        decode_attention(query, kv_cache, plan, 1.0 / math.sqrt(w.head_dim), output)
+    torch.cuda.synchronize()
+    ref, _ = ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, w.seq_lens)
+    err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
+    tol = 2e-3 if w.dtype == torch.float16 else 1.6e-2
+    print(f"[parity] vLLM decode {name}: max|out - ref| = {err:.3e} (tol {tol:.1e})", flush=True)
+    assert err <= tol
+
+
+def _grown(w, steps, spare_blocks):
+    """Block table (CPU, padded) and lengths of workload w after `steps` more tokens per request; new
+    blocks come from `spare_blocks` in request order."""
+    rows = [list(r) for r in w.rows]
+    lens = list(w.seq_lens)
+    spare = iter(spare_blocks)
+    for _ in range(steps):
+        for i in range(len(rows)):
+            if lens[i] % w.page_size == 0:
+                rows[i].append(next(spare))
+            lens[i] += 1
+    return rows, lens
+
+
+def _table(rows, width):
+    t = torch.zeros(len(rows), width, dtype=torch.int32)
+    for i, r in enumerate(rows):
+        t[i, :len(r)] = torch.tensor(r, dtype=torch.int32)
+    return t
+
+
+def test_advance_step_keeps_the_plan_right_on_cpu():
+    """After every in-place advance the plan, executed item by item by the oracle, gives dense
+    attention over the grown requests (c1: 8 requests x 288 tokens, so step 1 crosses a page)."""
+    w = workloads.make("c1", seed=5)
+    steps = 20
+    spare = list(range(w.num_blocks, w.num_blocks + 64))
+    width = w.padded_table().shape[1] + 2
+    meta = fake_metadata(w, torch.device("cpu"))
+    meta.block_tables_cpu = _table(w.rows, width)
+    meta.block_tables = meta.block_tables_cpu.clone()
+    plan = DecodePlan.from_metadata(meta)
+    gen = torch.Generator().manual_seed(1)
+    q = torch.randn(w.batch, 1, w.heads, w.head_dim, generator=gen)
+    k = torch.randn(w.num_blocks + 64, w.page_size, w.kv_heads, w.head_dim, generator=gen)
+    v = torch.randn(w.num_blocks + 64, w.page_size, w.kv_heads, w.head_dim, generator=gen)
+    in_place = 0
+    for step in range(1, steps + 1):
+        rows, lens = _grown(w, step, spare)
+        in_place += plan.advance_step(_table(rows, width))
+        assert plan.seq_lens == lens
+        if step in (1, 2, 16, 17, 20):
+            info = plan._ready_tree().kernel_info
+            listed = {key: [t.tolist() for t in getattr(info, key)] for key in
+                      ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs")}
+            listed["num_split_per_seq"] = info.num_split_per_seq.tolist()
+            out, lse = ao.run_plan_ref(listed, q, k, v)
+            ref, ref_lse = ao.paged_attention_ref(q, k, v, rows, lens)
+            assert (out - ref).abs().max().item() < 1e-5, step
+            assert (lse - ref_lse).abs().max().item() < 1e-5, step
+    assert in_place + plan.replans == steps
+    assert in_place >= steps - 2          # a full block row may force a fresh plan now and then
+
+
+@pytest.mark.gpu
+def test_advance_step_on_gpu():
+    print("[case] vLLM multi-step advance c2", flush=True)
+    dev = torch.device("cuda:0")
+    w = workloads.make("c2", seed=6)
+    steps = 18
+    spare = list(range(w.num_blocks, w.num_blocks + 2 * w.batch))
+    width = w.padded_table().shape[1] + 2
+    meta = fake_metadata(w, dev)
+    meta.block_tables_cpu = _table(w.rows, width)
+    meta.block_tables = meta.block_tables_cpu.to(dev)
+    plan = DecodePlan.from_metadata(meta)
+    gen = torch.Generator().manual_seed(2)
+    q = torch.randn(w.batch, 1, w.heads, w.head_dim, generator=gen).to(w.dtype)
+    k = torch.randn(w.num_blocks + 2 * w.batch, w.page_size, w.kv_heads, w.head_dim, generator=gen).to(w.dtype)
+    v = torch.randn(w.num_blocks + 2 * w.batch, w.page_size, w.kv_heads, w.head_dim, generator=gen).to(w.dtype)
+    kv_cache = torch.stack([k, v]).to(dev)
+    query = q.squeeze(1).to(dev)
+    output = torch.empty_like(query)
+    for step in range(1, steps + 1):
+        rows, lens = _grown(w, step, spare)
+        plan.advance_step(_table(rows, width))
+        decode_attention(query, kv_cache, plan, 1.0 / math.sqrt(w.head_dim), output)
+        if step in (1, 9, 18):
+            torch.cuda.synchronize()
+            ref, _ = ao.paged_attention_ref(q, k, v, rows, lens)
+            err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
+            print(f"[parity] advance step {step}: max|out - ref| = {err:.3e} (replans {plan.replans})", flush=True)
+            assert err <= 1.6e-2
