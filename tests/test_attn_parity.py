@@ -217,6 +217,44 @@ def test_page_sizes_and_tiny_boxes(page, dtype, heads):
     _assert_close(f"page {page}", out, lse, ref_out, ref_lse, dtype)
 
 
+def test_hip_graph_replay_matches_eager():
+    # both kernels of a call captured into a HIP graph (what a serving loop does with a decode step):
+    # every replay, with the program's own eager work between replays, must equal the eager result
+    print("[case] HIP graph capture and replay, c2", flush=True)
+    dev = _device()
+    w = workloads.make("c2", seed=7)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    scale = 1.0 / math.sqrt(w.head_dim)
+    q_static = q.clone()
+    out_graph = torch.zeros_like(q)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        prefix_attn_with_kvcache(q_static, k, v, tree, scale, out_graph)      # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        prefix_attn_with_kvcache(q_static, k, v, tree, scale, out_graph)
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    for trial in range(4):
+        q_new = torch.randn(q.shape, generator=gen).to(w.dtype).to(dev)
+        out_eager = torch.full_like(q, float("nan"))
+        prefix_attn_with_kvcache(q_new, k, v, tree, scale, out_eager)
+        torch.cuda.synchronize()
+        q_static.copy_(q_new)
+        out_graph.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph, out_eager), f"replay {trial} differs from the eager call"
+    ref_out, _ = _oracle(w, q_static, k, v)
+    assert (out_graph.float().cpu() - ref_out.float()).abs().max().item() <= TOL[w.dtype]
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
