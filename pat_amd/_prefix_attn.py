@@ -12,6 +12,7 @@ the HIP kernels of libpat_amd; there is no PyTorch fallback path.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 from typing import List, Optional, Sequence, Union
 
@@ -20,6 +21,9 @@ import torch
 
 from . import _lib
 from .prefix_tree import _NativeTree
+
+_LIB = _lib.load()   # raises when libpat_amd.so is missing: there is no other path
+_current_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)
 
 __all__ = ["prefix_attn_with_kvcache", "PrefixTreeCPP", "KernelInfo"]
 
@@ -226,14 +230,20 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
     return L
 
 
+def _raw_stream(index: int) -> int:
+    """Handle of torch's current stream on device `index` (the short way when torch offers it)."""
+    fast = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    return fast(index) if fast is not None else torch.cuda.current_stream(index).cuda_stream
+
+
 def _run(L: _Launch, device: torch.device) -> None:
-    lib = _lib.load()
     # scratch for the partial results, from torch's caching allocator on the current stream
     ws = torch.empty(L.need, dtype=torch.uint8, device=device)
     L.args.workspace = ws.data_ptr()
     L.args.workspace_bytes = L.need
-    stream = torch.cuda.current_stream(device).cuda_stream
-    _lib.check(lib.pat_fwd_launch(C.byref(L.args), C.c_void_p(stream)))
+    rc = _LIB.pat_fwd_launch(C.byref(L.args), C.c_void_p(_raw_stream(device.index)))
+    if rc:
+        _lib.check(rc)
 
 
 def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cache_paged: torch.Tensor,
@@ -272,7 +282,10 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
     out = vals["out"]
     for name, t in (("q", q), ("kcache", k_cache_paged), ("vcache", v_cache_paged)):
         _check(isinstance(t, torch.Tensor) and t.is_cuda, f"{name} must be on CUDA")
-    with torch.cuda.device(q.device):
+    # the kernels launch on the current HIP device: switch only when q lives elsewhere
+    index = q.device.index
+    guard = torch.cuda.device(index) if index != _current_device() else contextlib.nullcontext()
+    with guard:
         if is_tree:
             tree = vals["tree"]
             tree = getattr(tree, "tree", tree) if not isinstance(tree, PrefixTreeCPP) else tree
