@@ -234,6 +234,13 @@ typedef struct pat_fwd_geometry {
 } pat_fwd_geometry;
 int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out);
 
+/* Device self-test (no counterpart in the reference): runs a one-wave kernel on `hip_stream` that
+ * checks the lane-swap reductions and the transposed LDS read against their definitions - the
+ * instruction-level facts the split kernel is built on - and stores the number of mismatches in
+ * *failures (0 = all hold). Allocates 4 bytes of device memory and synchronises the stream: a
+ * diagnostic, not part of the decode path. */
+int pat_selftest_device(void* hip_stream, int32_t* failures);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -100,6 +100,7 @@ SYMBOLS = {
     "pat_fwd_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_launch": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
     "pat_fwd_geometry_of": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(FwdGeometry)]),
+    "pat_selftest_device": (C.c_int, [C.c_void_p, C.POINTER(C.c_int32)]),
 }
 
 _lib: Optional[C.CDLL] = None

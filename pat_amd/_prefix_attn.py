@@ -22,7 +22,6 @@ import torch
 from . import _lib
 from .prefix_tree import _NativeTree
 
-_LIB = _lib.load()   # raises when libpat_amd.so is missing: there is no other path
 _current_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)
 
 __all__ = ["prefix_attn_with_kvcache", "PrefixTreeCPP", "KernelInfo"]
@@ -241,7 +240,7 @@ def _run(L: _Launch, device: torch.device) -> None:
     ws = torch.empty(L.need, dtype=torch.uint8, device=device)
     L.args.workspace = ws.data_ptr()
     L.args.workspace_bytes = L.need
-    rc = _LIB.pat_fwd_launch(C.byref(L.args), C.c_void_p(_raw_stream(device.index)))
+    rc = _lib.load().pat_fwd_launch(C.byref(L.args), C.c_void_p(_raw_stream(device.index)))
     if rc:
         _lib.check(rc)
 

@@ -29,6 +29,7 @@ SOURCES = [
     "capi_fwd.hip",
     "hip/pat_split.hip",
     "hip/pat_merge.hip",
+    "hip/selftest.hip",
 ]
 
 COMMON = ["-std=c++17", "-O3", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",

@@ -255,6 +255,18 @@ def test_hip_graph_replay_matches_eager():
     assert (out_graph.float().cpu() - ref_out.float()).abs().max().item() <= TOL[w.dtype]
 
 
+def test_device_selftest_reports_no_mismatch():
+    # lane-swap reductions and the transposed LDS read behave as the split kernel assumes
+    print("[case] device self-test", flush=True)
+    import ctypes as C
+    from pat_amd import _lib
+    _device()
+    failures = C.c_int32(-1)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(_lib.load().pat_selftest_device(C.c_void_p(stream), C.byref(failures)))
+    assert failures.value == 0
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
