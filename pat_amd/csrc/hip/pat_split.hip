@@ -119,9 +119,14 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   for (int i = 1; i < kMaxBuckets; ++i) bi += (item >= p.item_begin[i]) ? 1 : 0;
   const BucketDev bk = p.bucket[bi];
   const int local = item - bk.item_begin;
-  const int chunk = local % bk.chunks;
-  const int box = local / bk.chunks;
-  if (box >= bk.num_boxes) return;
+  // chunk-major inside a bucket: all boxes' first chunks, then all second chunks, ... Workgroups
+  // are handed to the shader engines round-robin in launch order and the hand-out stalls while
+  // the engine whose turn it is is full, so work must not correlate with the launch index: in
+  // box-major order the filled chunks of short boxes recur with the period of the reserved
+  // chunks, land on the same engines every time and leave the others idle.
+  const int chunk = local / bk.num_boxes;
+  const int box = local - chunk * bk.num_boxes;
+  if (chunk >= bk.chunks) return;
 #ifdef PAT_TRACE
   const int wg = item * p.kv_heads + head;
 #endif
@@ -178,6 +183,14 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     const int last = (chunk == bk.chunks - 1) ? p.chunks_per_rank : chunk + 1;  // exclusive
     if ((shared_tiles || wave == 0) && g == 0 && my_slot0 >= 0)
       for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
+#ifdef PAT_TRACE
+    if (empty && p.trace && tid == 0) {
+      long long* t = p.trace + (long long)wg * 8;
+      const long long now = wall_clock64();
+      t[0] = tr[0]; t[1] = now; t[2] = now; t[3] = now; t[4] = now; t[5] = 0; t[6] = 0;
+      t[7] = ((long long)bi << 48) | ((long long)box << 24) | chunk;
+    }
+#endif
     if (empty) return;
   }
   const int t_end = (kv < t_begin + bk.chunk_tokens) ? kv : t_begin + bk.chunk_tokens;
