@@ -26,6 +26,9 @@ constexpr int kTargetWgsPerCU = 2;  // what fits at once: 2 workgroups of 4 wave
 constexpr int kMinChunk = 128;      // tokens
 constexpr int kMaxChunk = 2048;
 constexpr int kTallChunk = 256;
+constexpr int kTallChunkBusy = 768;          // tall chunk when the launch does not fit on the device at once
+constexpr int kResidentWgsPerCU = 3;
+constexpr int64_t kLeafChunkBytes = 256 << 10;  // K+V bytes per head of a short box's chunk in that case
 
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
@@ -135,6 +138,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
   if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
+  const bool env_chunk = chunk > 0, env_tall = tall > 0;
   if (chunk <= 0) {
     // whole multiples of 128 tokens: the 4 waves of a workgroup get the same number of steps,
     // and boxes a little longer than the average do not spill a few tokens into a second chunk
@@ -145,6 +149,30 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     // at least kTallChunk; longer when the tall boxes alone would still fill the device
     tall = ceil_div64(tall_work / (kTargetWgsPerCU * kNumCUs), 128) * 128;
     tall = std::max<int64_t>(kTallChunk, std::min<int64_t>(kMaxChunk, tall));
+  }
+  if (!env_chunk || !env_tall) {
+    // With the sizes above, does the launch fit on the device at once (3 workgroups per CU)? If
+    // not, workgroups start in launch order as others retire, and long ones that start late set
+    // the run time: short boxes then get chunks of at most 256 KB of K+V per head (finer grain,
+    // better packing); and when the launch is more than twice what fits, tall boxes get at least
+    // 768 tokens (fewer, longer workgroups: their partial rows are the expensive part once they
+    // are off the critical path).
+    auto count = [&](int64_t c_leaf, int64_t c_tall) {
+      int64_t n = 0;
+      for (int i = 0; i < a->num_buckets; ++i) {
+        const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+        const int64_t c = row_tiles(a->buckets[i].mnw[0]) > 1 ? c_tall : c_leaf;
+        n += (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, c)) * a->kv_heads;
+      }
+      return n;
+    };
+    const int64_t resident = (int64_t)kResidentWgsPerCU * kNumCUs;
+    if (!env_chunk && count(round_unit(chunk), round_unit(tall)) > resident) {
+      const int64_t leaf_cap = std::max<int64_t>(kMinChunk, kLeafChunkBytes / (2 * a->head_dim * 2) / 128 * 128);
+      chunk = std::min(chunk, leaf_cap);
+    }
+    if (!env_tall && count(round_unit(chunk), round_unit(tall)) > 2 * resident)
+      tall = std::max<int64_t>(tall, kTallChunkBusy);
   }
   g->chunk = (int)std::min(round_unit(chunk), cap);
   g->tall_chunk = (int)std::min(round_unit(tall), cap);
