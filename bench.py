@@ -151,6 +151,15 @@ def main() -> None:
             raise RuntimeError(_lib.last_error())
 
     def timed(launches, steps, warmup):
+        # an idle GPU starts at low clocks: run untimed until 30 ms have passed (matters for the
+        # workloads whose whole timed region is a few milliseconds), then the W warm-up steps
+        spin = time.perf_counter()
+        i = 0
+        while time.perf_counter() - spin < 0.03:
+            step(launches, i)
+            i += 1
+            if i % 64 == 0:
+                torch.cuda.synchronize()
         for i in range(warmup):
             step(launches, i)
         torch.cuda.synchronize()
