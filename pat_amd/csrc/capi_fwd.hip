@@ -39,6 +39,13 @@ inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = 
 // (16,128,1) for pages under 32 tokens, csrc/api.h:177-181).
 inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 2 : 4); }
 
+// Widest box (tokens) of a bucket whose workgroups serve one kv head per wave
+// (PAT_HEAD_PER_WAVE_TOKENS overrides; 0 switches the mode off).
+int64_t head_per_wave_tokens() {
+  if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_TOKENS")) return std::atoll(env);
+  return 256;
+}
+
 struct Geometry {
   int chunk = 0;             // tokens per workgroup, boxes of <= 16 rows
   int tall_chunk = 0;        // tokens per workgroup, boxes of 17..64 rows
@@ -46,6 +53,7 @@ struct Geometry {
   int num_slots = 0;
   int bucket_chunk[kMaxBuckets] = {0};
   int bucket_chunks[kMaxBuckets] = {0};
+  int bucket_heads_per_wg[kMaxBuckets] = {0};   // 1, or kWaves: one kv head per wave
   int64_t total_wgs = 0;
 };
 
@@ -187,11 +195,25 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     const int n = (int)std::max<int64_t>(1, ceil_div64(tok, c));
     g->bucket_chunk[i] = (int)c;
     g->bucket_chunks[i] = n;
+    g->bucket_heads_per_wg[i] = 1;
     g->chunks_per_rank = std::max(g->chunks_per_rank, n);
-    g->total_wgs += (int64_t)a->buckets[i].num_boxes * n * a->kv_heads;
+    g->total_wgs += (int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / g->bucket_heads_per_wg[i]);
+  }
+  // Buckets whose widest box is a few steps long leave most waves of a workgroup idle and pay the
+  // workgroup's fixed cost once per kv head: there each wave takes a kv head of its own and walks
+  // the box alone. Only when the launch has workgroups to spare (2 per CU or more): a small launch
+  // is faster with every wave busy.
+  if (g->total_wgs >= 2 * kNumCUs && a->kv_heads % kWaves == 0) {
+    for (int i = 0; i < a->num_buckets; ++i) {
+      const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+      if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= head_per_wave_tokens()) {
+        g->bucket_heads_per_wg[i] = kWaves;
+        g->total_wgs -= (int64_t)a->buckets[i].num_boxes * (a->kv_heads - a->kv_heads / kWaves);
+      }
+    }
   }
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
-  if (g->total_wgs / a->kv_heads > (int64_t)kGridItemsY * 65535)
+  if (g->total_wgs > (int64_t)kGridX * 65535 || g->total_wgs >= INT32_MAX)
     return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   // the kernels index partial rows with 32-bit integers
   if ((int64_t)a->batch * a->heads * g->num_slots >= ((int64_t)1 << 31))
@@ -291,10 +313,11 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
       d.chunk_tokens = g.bucket_chunk[i];
       d.chunks = g.bucket_chunks[i];
       d.row_tiles = row_tiles(b.mnw[0]);
+      d.heads_per_wg = g.bucket_heads_per_wg[i];
       d.item_begin = (int32_t)items;
       sp.item_begin[nb] = (int32_t)items;
       ++nb;
-      items += (int64_t)b.num_boxes * d.chunks;
+      items += (int64_t)b.num_boxes * d.chunks * (args->kv_heads / d.heads_per_wg);
     }
     sp.num_buckets = nb;
     sp.total_items = (int32_t)items;

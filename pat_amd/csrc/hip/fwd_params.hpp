@@ -8,7 +8,7 @@ constexpr int kMaxBuckets = 12;    // the reference dispatches 12 tile shapes (s
 constexpr int kWaves = 4;          // waves per split-kernel workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kStepTokens = 32;    // KV tokens one wave consumes per loop iteration
-constexpr int kGridItemsY = 32768;  // work items per grid.y slice (grid.z counts slices)
+constexpr int kGridX = 1 << 20;     // workgroups per grid.x slice (grid.y counts slices)
 constexpr int kMaxChunkPages = 128; // page ids of a chunk: two per lane of a wave
 
 // One tile bucket as the split kernel sees it.
@@ -26,9 +26,9 @@ struct BucketDev {
   int32_t max_blocks;    // valid block_table columns
   int32_t chunk_tokens;  // KV tokens per workgroup (multiple of 32 and of page_size)
   int32_t chunks;        // workgroups along the KV axis reserved per box
-  int32_t item_begin;    // first work item (box, chunk) of this bucket
+  int32_t item_begin;    // first workgroup of this bucket in the launch (workgroups = items x head groups)
   int32_t row_tiles;     // 16-row tiles per box: 1 = KV steps split over waves, 2/4 = one wave per tile
-  int32_t pad_;
+  int32_t heads_per_wg;  // 1, or kWaves for buckets of very short boxes: wave w serves kv head h0 + w alone
 };
 
 struct SplitParams {
@@ -45,7 +45,7 @@ struct SplitParams {
   int32_t chunks_per_rank;  // slots reserved per CTA_rank
   int32_t num_slots;        // max_split_per_seq * chunks_per_rank
   int32_t max_split;
-  int32_t total_items;      // work items (box, chunk) over all buckets; the grid is (kv_heads, items)
+  int32_t total_items;      // workgroups over all buckets: (box, chunk) items x head groups, head group fastest
   float scale_log2;         // softmax_scale * log2(e)
   int32_t num_buckets;
   uint32_t hpp_magic;       // ceil(2^32 / (page_size / 16)): h / (page_size / 16) == umulhi(h, hpp_magic) for h < 2^16; unused when page_size / 16 is a power of two

@@ -112,13 +112,20 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   // grid = (kv heads, work items): the head is the fastest-varying part of the dispatch order.
   // The bucket is found from a table at fixed kernel-argument offsets and its descriptor is
   // fetched whole, so the decode costs two scalar-memory round trips, not one per field.
-  const int head = blockIdx.x;
-  const int item = blockIdx.z * kGridItemsY + blockIdx.y;   // past the last item: lands past the last box
+  const int wg_id = blockIdx.y * kGridX + blockIdx.x;   // past the last workgroup: lands past the last box
   int bi = 0;
 #pragma unroll
-  for (int i = 1; i < kMaxBuckets; ++i) bi += (item >= p.item_begin[i]) ? 1 : 0;
+  for (int i = 1; i < kMaxBuckets; ++i) bi += (wg_id >= p.item_begin[i]) ? 1 : 0;
   const BucketDev bk = p.bucket[bi];
-  const int local = item - bk.item_begin;
+  // head group fastest: consecutive workgroups (dealt to the XCDs round-robin) serve consecutive
+  // kv heads of one item. Buckets of very short boxes give each wave a kv head of its own.
+  const bool head_per_wave = bk.heads_per_wg > 1;
+  const int head_groups = p.kv_heads / bk.heads_per_wg;
+  const int wg_local = wg_id - bk.item_begin;
+  const int local = wg_local / head_groups;
+  // (uniform over the wave: kept in a scalar register so that address arithmetic stays scalar)
+  const int head = __builtin_amdgcn_readfirstlane(
+      (wg_local - local * head_groups) * bk.heads_per_wg + (head_per_wave ? (int)(threadIdx.x >> 6) : 0));
   // chunk-major inside a bucket: all boxes' first chunks, then all second chunks, ... Workgroups
   // are handed to the shader engines round-robin in launch order and the hand-out stalls while
   // the engine whose turn it is is full, so work must not correlate with the launch index: in
@@ -128,7 +135,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const int box = local - chunk * bk.num_boxes;
   if (chunk >= bk.chunks) return;
 #ifdef PAT_TRACE
-  const int wg = item * p.kv_heads + head;
+  const int wg = wg_id;
 #endif
 
   // Boxes of up to 16 rows: the 4 waves split the chunk's steps, each on wave-private tiles.
@@ -181,7 +188,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     const bool empty = t_begin >= kv;
     const int first = empty ? chunk : chunk + 1;
     const int last = (chunk == bk.chunks - 1) ? p.chunks_per_rank : chunk + 1;  // exclusive
-    if ((shared_tiles || wave == 0) && g == 0 && my_slot0 >= 0)
+    if ((shared_tiles || head_per_wave || wave == 0) && g == 0 && my_slot0 >= 0)
       for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
 #ifdef PAT_TRACE
     if (empty && p.trace && tid == 0) {
@@ -426,22 +433,25 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         for (int kk = 0; kk < KK; ++kk) kd[a][kk] = *(const u32x4*)(kb + ko + kk * 64);
       }
     };
+    // steps of this wave: every kWaves-th one of the chunk, or, with a kv head per wave, all of them
+    const int step0 = head_per_wave ? 0 : wave;
+    const int stride = head_per_wave ? 1 : kWaves;
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
-      if (wave + d * kWaves < nsteps) {
-        fetch_v(wave + d * kWaves, vring[d]);
-        fetch_k(wave + d * kWaves, kring[d]);
+      if (step0 + d * stride < nsteps) {
+        fetch_v(step0 + d * stride, vring[d]);
+        fetch_k(step0 + d * stride, kring[d]);
       }
 #ifdef PAT_TRACE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     PAT_STAMP(2);
 #endif
-    for (int st0 = wave; st0 < nsteps; st0 += DEPTH * kWaves) {
+    for (int st0 = step0; st0 < nsteps; st0 += DEPTH * stride) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
-        const int st = st0 + d * kWaves;
+        const int st = st0 + d * stride;
         if (st >= nsteps) break;
-        const int nxt = st + DEPTH * kWaves;
+        const int nxt = st + DEPTH * stride;
         const bool more = nxt < nsteps;
         // V tile -> this wave's LDS region, row-major with padded rows; its registers are free
         // again at once and take the ring's next V tile
@@ -457,6 +467,17 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     PAT_STAMP(3);
     l_run = sum_xor32(sum_xor16(l_run));
 
+    if (head_per_wave) {
+      // the wave has seen the whole chunk of its head: its rows go out as they are
+      if (my_slot0 >= 0) {
+        const int64_t prow = (int64_t)my_slot0 + chunk;
+        const float inv = 1.f / l_run;
+        float* dst = p.o_part + prow * D + g * 4;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
+        if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+      }
+    } else {
     // combine the 4 waves' states through LDS and write the partial
     float* cbuf = (float*)smem;
     const int crow = tid >> 4;                 // row this thread finalises
@@ -494,6 +515,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       if ((tid & 15) == 0)
         p.lse_part[prow] = (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f;
     }
+    }   // combine
   }
 #ifdef PAT_TRACE
   if (p.trace && tid == 0) {
@@ -515,9 +537,8 @@ hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const Split
   void (*fn)(const SplitParams);
   if (bf16) fn = head_dim == 64 ? pat_split_kernel<__bf16, 64> : pat_split_kernel<__bf16, 128>;
   else fn = head_dim == 64 ? pat_split_kernel<_Float16, 64> : pat_split_kernel<_Float16, 128>;
-  const unsigned items = (unsigned)params.total_items;
-  const dim3 grid((unsigned)params.kv_heads, items < (unsigned)kGridItemsY ? items : (unsigned)kGridItemsY,
-                  (items + kGridItemsY - 1) / kGridItemsY);
+  const unsigned wgs = (unsigned)params.total_items;
+  const dim3 grid(wgs < (unsigned)kGridX ? wgs : (unsigned)kGridX, (wgs + kGridX - 1) / kGridX);
   hipLaunchKernelGGL(fn, grid, dim3(kThreads), 0, stream, params);
   return hipGetLastError();
 }
