@@ -9,10 +9,12 @@
 // those tokens plus LSE = max + ln(sum) (csrc/softmax.h:169-188).
 //
 // Mapping to the hardware (this kernel's own design):
-//  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each; grid = (kv heads,
-//    items), so the kv-head is the fastest-varying part of the dispatch order: workgroups are
-//    dealt to the 8 XCDs round-robin, so with 8 kv-heads XCD x serves head x and boxes that
-//    share KV pages (the boxes of one prefix node) find them in that XCD's L2.
+//  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each, launched as a flat
+//    list with the kv-head fastest: workgroups are dealt to the 8 XCDs round-robin, so with 8
+//    kv-heads XCD x serves head x and boxes that share KV pages (the boxes of one prefix node)
+//    find them in that XCD's L2. Inside a bucket the list is chunk-major (see the decode below).
+//  * buckets of very short boxes: one workgroup serves 4 kv heads, one per wave, each wave
+//    walking its head's steps alone (no combine).
 //  * boxes of up to 16 rows (one MFMA row tile): each wave owns every 4th 32-token step of
 //    the chunk on wave-private tiles and runs an independent online softmax; the 4 states are
 //    combined through LDS at the end. K rows are the MFMA A operand of S^T = K.Q^T, so a lane
@@ -109,7 +111,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const int n = lane & 15;   // index inside the group
 
   // ---- which (bucket, box, chunk, kv-head) is this workgroup? ---------------------------
-  // grid = (kv heads, work items): the head is the fastest-varying part of the dispatch order.
+  // a flat list of workgroups, head (group) fastest inside an item.
   // The bucket is found from a table at fixed kernel-argument offsets and its descriptor is
   // fetched whole, so the decode costs two scalar-memory round trips, not one per field.
   const int wg_id = blockIdx.y * kGridX + blockIdx.x;   // past the last workgroup: lands past the last box
