@@ -138,12 +138,13 @@ def main() -> None:
             L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), ws.numel()
         return launches, ws
 
-    pat_kw = dict(num_split_per_seq=info.num_split_per_seq, query_tables=info.q_tables,
-                  block_tables=info.block_tables, num_seqs_per_CTAs=info.num_seqs_per_CTAs,
-                  CTA_ranks=info.CTA_ranks, kv_in_CTAs=info.kv_in_CTAs, MNW=info.MNWs,
+    lt = info.launch_tables()   # what prefix_attn_with_kvcache(tree=...) hands to the kernels
+    pat_kw = dict(num_split_per_seq=info.num_split_per_seq, query_tables=lt["q_tables"],
+                  block_tables=lt["block_tables"], num_seqs_per_CTAs=lt["num_seqs_per_CTAs"],
+                  CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=info.MNWs,
                   max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                   max_blocks_in_CTA=info.max_blocks_in_CTA)
-    pat_launches, pat_ws = prepare(pat_kw, info.slot_tables)
+    pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"])
 
     def step(launches, i):
         rc = lib.pat_fwd_launch(C.byref(launches[i % copies].args), C.c_void_p(stream))

@@ -51,6 +51,28 @@ class KernelInfo:
         self.max_seqs_in_CTA = 0
         self.max_blocks_in_CTA = 0
         self._launch_cache: dict = {}
+        # Launch copies of the per-bucket tables with every bucket's boxes ordered longest first
+        # (what the kernels are given; the tables above keep the scheduler's order). Workgroups
+        # start in launch order and are dealt round-robin to the CUs, so this order gives every
+        # CU a similar mix and keeps long boxes from starting last.
+        self._launch_tables: Optional[dict] = None
+        self._launch_order: List[torch.Tensor] = []   # per bucket: launch row -> scheduler row
+
+    _PER_BOX = ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "slot_tables")
+
+    def _sort_for_launch(self) -> None:
+        self._launch_order = [torch.argsort(kv, descending=True, stable=True) for kv in self.kv_in_CTAs]
+        self._launch_tables = {
+            name: [t[order].contiguous() for t, order in zip(getattr(self, name), self._launch_order)]
+            for name in self._PER_BOX if getattr(self, name)}
+        self._launch_cache.clear()
+
+    def launch_tables(self) -> dict:
+        """The per-bucket tables as the kernels get them (longest box first); the scheduler-order
+        tables when no launch copies exist."""
+        if self._launch_tables is not None:
+            return self._launch_tables
+        return {name: getattr(self, name) for name in self._PER_BOX}
 
     def to_gpu(self, device: Union[torch.device, str]) -> None:
         """Copies every plan tensor to `device` (asynchronously where the source is pinned)."""
@@ -66,6 +88,9 @@ class KernelInfo:
         self.kv_in_CTAs = [move(t) for t in self.kv_in_CTAs]
         self.slot_tables = [move(t) for t in self.slot_tables]
         self.num_split_per_seq = move(self.num_split_per_seq)
+        if self._launch_tables is not None:
+            self._launch_tables = {name: [move(t) for t in ts] for name, ts in self._launch_tables.items()}
+            self._launch_order = [move(t) for t in self._launch_order]
         self._launch_cache.clear()
 
     @classmethod
@@ -94,6 +119,7 @@ class KernelInfo:
         ki.max_split_per_seq = view.max_split_per_seq
         ki.max_seqs_in_CTA = view.max_seqs_in_box
         ki.max_blocks_in_CTA = view.max_blocks_in_box
+        ki._sort_for_launch()
         return ki
 
 
@@ -294,10 +320,11 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                    q.dtype, float(vals["softmax_scale"]), None if lse is None else lse.data_ptr())
             L = info._launch_cache.get(key)
             if L is None:
-                L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, info.q_tables,
-                             info.block_tables, info.num_seqs_per_CTAs, info.CTA_ranks, info.kv_in_CTAs,
+                lt = info.launch_tables()
+                L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, lt["q_tables"],
+                             lt["block_tables"], lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"],
                              info.MNWs, info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
-                             vals["softmax_scale"], out, lse, info.slot_tables)
+                             vals["softmax_scale"], out, lse, lt.get("slot_tables"))
                 if len(info._launch_cache) >= 256:
                     info._launch_cache.clear()
                 info._launch_cache[key] = L

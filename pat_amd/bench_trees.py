@@ -63,8 +63,9 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
     tree.pack_schedule(None, heads // kv_heads, kv_heads)
     info = tree.kernel_info
     info.to_gpu(dev)
-    aware = dict(num_split_per_seq=info.num_split_per_seq, query_tables=info.q_tables, block_tables=info.block_tables,
-                 num_seqs_per_CTAs=info.num_seqs_per_CTAs, CTA_ranks=info.CTA_ranks, kv_in_CTAs=info.kv_in_CTAs,
+    lt = info.launch_tables()   # what prefix_attn_with_kvcache(tree=...) hands to the kernels
+    aware = dict(num_split_per_seq=info.num_split_per_seq, query_tables=lt["q_tables"], block_tables=lt["block_tables"],
+                 num_seqs_per_CTAs=lt["num_seqs_per_CTAs"], CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"],
                  MNW=info.MNWs, max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                  max_blocks_in_CTA=info.max_blocks_in_CTA)
     oblivious = workloads.oblivious_plan(w, dev)
@@ -93,7 +94,7 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / iters * 1e3
 
-    made_a, keep_a = launches(aware, info.slot_tables)
+    made_a, keep_a = launches(aware, lt["slot_tables"])
     t_aware = timed(made_a)
     made_o, keep_o = launches(oblivious, None)
     t_obl = timed(made_o)

@@ -49,6 +49,7 @@ class DecodePlan:
     replans: int = 0                           # times advance_step had to plan afresh
     _tails: Any = None                         # per request (bucket, box) of the item holding its tail
     _tail_kv: Any = None
+    _launch_row: Any = None                    # per bucket: scheduler row -> launch row
 
     @classmethod
     def from_metadata(cls, meta: Any) -> Optional["DecodePlan"]:
@@ -96,6 +97,7 @@ class DecodePlan:
         self.tree = AsyncTree(block_size=self.block_size, seq_lens=list(self.seq_lens), table=table_cpu, MNWs=None,
                               HRatio=self.nheads // self.nheads_kv, kvHead=self.nheads_kv, device=device)
         self._tails = None
+        self._launch_row = None
         self.replans += 1
 
     def advance_step(self, block_tables_cpu: torch.Tensor) -> bool:
@@ -128,15 +130,28 @@ class DecodePlan:
             ids.append(int(table_cpu[s, n_old // bs]))
         self._tail_kv += 1
         device = info.num_split_per_seq.device
-        for b in range(len(info.MNWs)):
-            boxes = self._tails[self._tails[:, 0] == b, 1]
-            if len(boxes):
-                info.kv_in_CTAs[b].index_add_(0, torch.as_tensor(boxes, device=device),
-                                              torch.ones(len(boxes), dtype=torch.int32, device=device))
-            if b in new_blocks:
-                where, ids = new_blocks[b]
-                info.block_tables[b].view(-1).index_copy_(0, torch.as_tensor(where, device=device),
-                                                          torch.as_tensor(ids, dtype=torch.int32, device=device))
+        # the tables the kernels read (boxes in launch order) and, so that they keep describing the
+        # same plan, the scheduler-order tables
+        launch = info.launch_tables()
+        targets = [(info.kv_in_CTAs, info.block_tables, None)]
+        if launch["kv_in_CTAs"] is not info.kv_in_CTAs:
+            if self._launch_row is None:
+                self._launch_row = [torch.argsort(order).cpu().numpy() for order in info._launch_order]
+            targets.append((launch["kv_in_CTAs"], launch["block_tables"], self._launch_row))
+        for kvs, tables, row_of in targets:
+            for b in range(len(info.MNWs)):
+                boxes = self._tails[self._tails[:, 0] == b, 1]
+                width = tables[b].shape[1]
+                if len(boxes):
+                    rows = boxes if row_of is None else row_of[b][boxes]
+                    kvs[b].index_add_(0, torch.as_tensor(rows, device=device),
+                                      torch.ones(len(rows), dtype=torch.int32, device=device))
+                if b in new_blocks:
+                    where, ids = new_blocks[b]
+                    if row_of is not None:
+                        where = [int(row_of[b][w // width]) * width + w % width for w in where]
+                    tables[b].view(-1).index_copy_(0, torch.as_tensor(where, device=device),
+                                                   torch.as_tensor(ids, dtype=torch.int32, device=device))
         return True
 
 

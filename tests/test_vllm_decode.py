@@ -118,6 +118,11 @@ def test_advance_step_keeps_the_plan_right_on_cpu():
             listed = {key: [t.tolist() for t in getattr(info, key)] for key in
                       ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs")}
             listed["num_split_per_seq"] = info.num_split_per_seq.tolist()
+            launch = info.launch_tables()       # the kernels' copies (longest box first) grew alike
+            for b, order in enumerate(info._launch_order):
+                assert torch.equal(launch["kv_in_CTAs"][b], info.kv_in_CTAs[b][order])
+                assert torch.equal(launch["block_tables"][b], info.block_tables[b][order])
+                assert (launch["kv_in_CTAs"][b][:-1] >= launch["kv_in_CTAs"][b][1:] - step).all()
             out, lse = ao.run_plan_ref(listed, q, k, v)
             ref, ref_lse = ao.paged_attention_ref(q, k, v, rows, lens)
             assert (out - ref).abs().max().item() < 1e-5, step
