@@ -28,7 +28,6 @@ constexpr int kMaxChunk = 2048;
 constexpr int kTallChunk = 256;
 constexpr int kTallChunkBusy = 768;          // tall chunk when the launch does not fit on the device at once
 constexpr int kResidentWgsPerCU = 3;
-constexpr int64_t kLeafChunkBytes = 256 << 10;  // K+V bytes per head of a short box's chunk in that case
 
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
@@ -41,9 +40,9 @@ inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 
 
 // Widest box (tokens) of a bucket whose workgroups serve one kv head per wave
 // (PAT_HEAD_PER_WAVE_TOKENS overrides; 0 switches the mode off).
-int64_t head_per_wave_tokens() {
+int64_t head_per_wave_tokens(bool oversubscribed) {
   if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_TOKENS")) return std::atoll(env);
-  return 256;
+  return oversubscribed ? 256 : 128;
 }
 
 struct Geometry {
@@ -146,7 +145,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
   if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
-  const bool env_chunk = chunk > 0, env_tall = tall > 0;
+  const bool env_tall = tall > 0;
   if (chunk <= 0) {
     // whole multiples of 128 tokens: the 4 waves of a workgroup get the same number of steps,
     // and boxes a little longer than the average do not spill a few tokens into a second chunk
@@ -158,28 +157,23 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     tall = ceil_div64(tall_work / (kTargetWgsPerCU * kNumCUs), 128) * 128;
     tall = std::max<int64_t>(kTallChunk, std::min<int64_t>(kMaxChunk, tall));
   }
-  if (!env_chunk || !env_tall) {
-    // With the sizes above, does the launch fit on the device at once (3 workgroups per CU)? If
-    // not, workgroups start in launch order as others retire, and long ones that start late set
-    // the run time: short boxes then get chunks of at most 256 KB of K+V per head (finer grain,
-    // better packing); and when the launch is more than twice what fits, tall boxes get at least
-    // 768 tokens (fewer, longer workgroups: their partial rows are the expensive part once they
-    // are off the critical path).
-    auto count = [&](int64_t c_leaf, int64_t c_tall) {
-      int64_t n = 0;
-      for (int i = 0; i < a->num_buckets; ++i) {
-        const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-        const int64_t c = row_tiles(a->buckets[i].mnw[0]) > 1 ? c_tall : c_leaf;
-        n += (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, c)) * a->kv_heads;
-      }
-      return n;
-    };
-    const int64_t resident = (int64_t)kResidentWgsPerCU * kNumCUs;
-    if (!env_chunk && count(round_unit(chunk), round_unit(tall)) > resident) {
-      const int64_t leaf_cap = std::max<int64_t>(kMinChunk, kLeafChunkBytes / (2 * a->head_dim * 2) / 128 * 128);
-      chunk = std::min(chunk, leaf_cap);
+  if (!env_tall) {
+    // Does the launch fit on the device at once (3 workgroups per CU)? When it is well past that,
+    // workgroups start in launch order as others retire and the tall boxes are off the critical
+    // path: they then get at least 768 tokens per workgroup (fewer, longer workgroups: their
+    // 16..32 KB of partial rows each are the expensive part). Short boxes keep their size: with
+    // the launch tables ordered longest first, finer chunks no longer pack better.
+    int64_t n = 0, n_tall = 0;
+    for (int i = 0; i < a->num_buckets; ++i) {
+      const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+      const bool is_tall = row_tiles(a->buckets[i].mnw[0]) > 1;
+      const int64_t c = is_tall ? round_unit(tall) : round_unit(chunk);
+      const int64_t wgs = (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, c)) * a->kv_heads;
+      n += wgs;
+      if (is_tall) n_tall += wgs;
     }
-    if (!env_tall && count(round_unit(chunk), round_unit(tall)) > 2 * resident)
+    // (a handful of tall boxes stays finely cut: there the tall chain is the critical path)
+    if (2 * n > 3 * (int64_t)kResidentWgsPerCU * kNumCUs && n_tall >= kNumCUs)
       tall = std::max<int64_t>(tall, kTallChunkBusy);
   }
   g->chunk = (int)std::min(round_unit(chunk), cap);
@@ -204,9 +198,12 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   // the box alone. Only when the launch has workgroups to spare (2 per CU or more): a small launch
   // is faster with every wave busy.
   if (g->total_wgs >= 2 * kNumCUs && a->kv_heads % kWaves == 0) {
+    // up to 256 tokens when the launch does not fit on the device at once, up to 128 when it
+    // does (every workgroup is resident from the start and the longest chain sets the time)
+    const int64_t limit = head_per_wave_tokens(g->total_wgs > (int64_t)kResidentWgsPerCU * kNumCUs);
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-      if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= head_per_wave_tokens()) {
+      if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= limit) {
         g->bucket_heads_per_wg[i] = kWaves;
         g->total_wgs -= (int64_t)a->buckets[i].num_boxes * (a->kv_heads - a->kv_heads / kWaves);
       }
