@@ -271,6 +271,27 @@ def _run(L: _Launch, device: torch.device) -> None:
         _lib.check(rc)
 
 
+_TABLE_LAUNCHES: dict = {}
+
+
+def _table_key(q, k, v, out, lse, vals, slots):
+    """Identity of a table-form call: every tensor's address and layout plus the scalars. None when
+    the arguments are not what a well-formed call passes (the full checks then raise)."""
+    try:
+        def ident(t):
+            return (t.data_ptr(), tuple(t.shape), t.stride())
+        def small(t):   # plan tensors: 1-D, or 2-D with contiguous rows (checked when the launch is built)
+            return (t.data_ptr(), t.numel(), t.stride(0))
+        lists = tuple(tuple(small(t) for t in vals[name]) for name in
+                      ("query_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs"))
+        return (ident(q), ident(k), ident(v), ident(out), q.dtype, None if lse is None else ident(lse),
+                small(vals["num_split_per_seq"]), lists, tuple(tuple(m) for m in vals["MNW"]),
+                int(vals["max_split_per_seq"]), int(vals["max_seqs_in_CTA"]), int(vals["max_blocks_in_CTA"]),
+                float(vals["softmax_scale"]), None if not slots else tuple(small(t) for t in slots))
+    except (AttributeError, TypeError, ValueError):
+        return None
+
+
 def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cache_paged: torch.Tensor,
                              *rest, **kw) -> None:
     """Prefix-aware decode attention over a paged KV cache; writes `out` in place.
@@ -329,8 +350,19 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                     info._launch_cache.clear()
                 info._launch_cache[key] = L
         else:
-            L = _prepare(q, k_cache_paged, v_cache_paged, vals["num_split_per_seq"], vals["query_tables"],
-                         vals["block_tables"], vals["num_seqs_per_CTAs"], vals["CTA_ranks"], vals["kv_in_CTAs"],
-                         vals["MNW"], vals["max_split_per_seq"], vals["max_seqs_in_CTA"],
-                         vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse, slots)
+            # the prepared launch is kept per set of tensors: a decode step calls this once per layer
+            # with the same plan, and building the argument block costs more than the kernels of a
+            # small batch take. The key holds what the block was built from (addresses and
+            # layouts); the tensors' contents are read by the kernels at every call.
+            key = _table_key(q, k_cache_paged, v_cache_paged, out, lse, vals, slots)
+            L = _TABLE_LAUNCHES.get(key) if key is not None else None
+            if L is None:
+                L = _prepare(q, k_cache_paged, v_cache_paged, vals["num_split_per_seq"], vals["query_tables"],
+                             vals["block_tables"], vals["num_seqs_per_CTAs"], vals["CTA_ranks"], vals["kv_in_CTAs"],
+                             vals["MNW"], vals["max_split_per_seq"], vals["max_seqs_in_CTA"],
+                             vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse, slots)
+                if key is not None:
+                    if len(_TABLE_LAUNCHES) >= 64:
+                        _TABLE_LAUNCHES.clear()
+                    _TABLE_LAUNCHES[key] = L
         _run(L, q.device)
