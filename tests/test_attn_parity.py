@@ -267,6 +267,42 @@ def test_device_selftest_reports_no_mismatch():
     assert failures.value == 0
 
 
+@pytest.mark.parametrize("heads,dtype", [((32, 8), torch.bfloat16), ((16, 16), torch.float16)])
+def test_large_ragged_batch_all_launch_modes(heads, dtype):
+    # a launch several times what fits on the device at once: short private tails (one kv head per
+    # wave), mid-size shared nodes, a few long shared roots read by many 64-row boxes, boxes sorted
+    # longest first for the launch
+    print(f"[case] large ragged batch heads={heads} {dtype}", flush=True)
+    import random
+    dev = _device()
+    r = random.Random(heads[0])
+    next_block = [0]
+
+    def blocks(n):
+        out = list(range(next_block[0], next_block[0] + n)); next_block[0] += n
+        return out
+
+    rows, lens = [], []
+    for _ in range(3):
+        root = blocks(r.randint(40, 90))               # 640..1440 shared tokens
+        for _ in range(r.randint(6, 10)):
+            mid = root + blocks(r.randint(2, 20))
+            for _ in range(r.randint(4, 24)):
+                row = mid + blocks(r.randint(1, 14))
+                rows.append(row)
+                lens.append(len(row) * 16 - r.randint(0, 15))
+    order = list(range(len(rows))); r.shuffle(order)
+    rows, lens = [rows[i] for i in order], [lens[i] for i in order]
+    perm = list(range(next_block[0])); r.shuffle(perm)
+    rows = [[perm[x] for x in row] for row in rows]
+    w = workloads.Workload("large", heads[0], heads[1], 128, dtype, 16, lens, rows, next_block[0], 0, 21)
+    print(f"        {w.batch} requests, {next_block[0]} blocks", flush=True)
+    q, k, v = w.tensors(dev)
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("large ragged", out, lse, ref_out, ref_lse, dtype)
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
