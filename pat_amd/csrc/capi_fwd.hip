@@ -180,6 +180,15 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   g->tall_chunk = (int)std::min(round_unit(tall), cap);
   g->chunks_per_rank = 1;
   g->total_wgs = 0;
+  int64_t kind_tall_wgs = 0, kind_short_wgs = 0;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const bool is_tall = row_tiles(a->buckets[i].mnw[0]) > 1;
+    const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+    const int64_t wgs = (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, is_tall ? g->tall_chunk : g->chunk)) * a->kv_heads;
+    (is_tall ? kind_tall_wgs : kind_short_wgs) += wgs;
+  }
+  int equalize = -1;   // PAT_EQUALIZE_CHUNKS=0/1 overrides the rule below (tuning aid)
+  if (const char* env = std::getenv("PAT_EQUALIZE_CHUNKS")) equalize = std::atoi(env) != 0;
   for (int i = 0; i < a->num_buckets; ++i) {
     const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
     int64_t c = row_tiles(a->buckets[i].mnw[0]) > 1 ? g->tall_chunk : g->chunk;
@@ -187,6 +196,13 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     if (ceil_div64(tok, c) > kMaxChunksPerRank)
       return fail(PAT_ERR_INVALID, "a box spans more KV blocks than one launch supports");
     const int n = (int)std::max<int64_t>(1, ceil_div64(tok, c));
+    // Same number of chunks, equal lengths (the widest box is cut into n even pieces instead of
+    // n - 1 full ones and a remainder) when the boxes of this kind are all resident from the
+    // start: the longest workgroup then sets when they are done. When they start in waves, the
+    // remainders, which the chunk-major order launches last, make the shorter tail.
+    const int64_t kind_wgs = row_tiles(a->buckets[i].mnw[0]) > 1 ? kind_tall_wgs : kind_short_wgs;
+    if (equalize == 1 || (equalize < 0 && kind_wgs <= (int64_t)kResidentWgsPerCU * kNumCUs))
+      c = std::min(c, round_unit(ceil_div64(tok, n)));
     g->bucket_chunk[i] = (int)c;
     g->bucket_chunks[i] = n;
     g->bucket_heads_per_wg[i] = 1;
