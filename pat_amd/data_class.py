@@ -175,6 +175,22 @@ class KernelInfo:
     # partial results by this ordinal instead of by CTA_rank.
     slot_tables: Any = field(default_factory=list)
 
+    def sort_for_launch(self) -> None:
+        """Not in the reference: orders every bucket's items longest first (stable), on the list
+        form, i.e. before `to_tensor`. The kernels start work items in table order, and the table
+        form of `prefix_attn_with_kvcache` launches the tables as they are given; longest first
+        keeps long items from starting last. The plan stays the same plan: rows of one bucket are
+        independent work items."""
+        per_box = [self.q_tables, self.block_tables, self.num_seqs_per_CTAs, self.CTA_ranks, self.kv_in_CTAs]
+        if self.slot_tables:
+            per_box.append(self.slot_tables)
+        if any(isinstance(t, torch.Tensor) for col in per_box for t in col):
+            raise ValueError("sort_for_launch() works on the list form: call it before to_tensor()")
+        for b, kv in enumerate(self.kv_in_CTAs):
+            order = sorted(range(len(kv)), key=kv.__getitem__, reverse=True)
+            for col in per_box:
+                col[b] = [col[b][i] for i in order]
+
     def to_tensor(self, device) -> None:
         def vectors(cols: Iterable) -> list:
             return [c if isinstance(c, torch.Tensor) else _vector(c, device) for c in cols]

@@ -57,3 +57,24 @@ def test_forward_refuses_cpu_tensors():
         raise AssertionError("expected a device check to fail")
     except RuntimeError as e:
         assert "must be on CUDA" in str(e)
+
+
+def test_python_plan_sort_for_launch_permutes_rows_only():
+    from pat_amd import workloads
+    w = workloads.make("c2")
+    tree = prefix_attn.PrefixTree(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.rows)
+    ki = tree.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+    before = [sorted(zip(map(tuple, ki.q_tables[b]), map(tuple, ki.block_tables[b]), ki.num_seqs_per_CTAs[b],
+                         ki.CTA_ranks[b], ki.kv_in_CTAs[b])) for b in range(len(ki.MNWs))]
+    ki.sort_for_launch()
+    after = [sorted(zip(map(tuple, ki.q_tables[b]), map(tuple, ki.block_tables[b]), ki.num_seqs_per_CTAs[b],
+                        ki.CTA_ranks[b], ki.kv_in_CTAs[b])) for b in range(len(ki.MNWs))]
+    assert before == after                                       # the same items
+    assert all(list(kv) == sorted(kv, reverse=True) for kv in ki.kv_in_CTAs)
+    ki.to_tensor("cpu")
+    try:
+        ki.sort_for_launch()
+        raise AssertionError("expected the tensor form to be refused")
+    except ValueError as e:
+        assert "before to_tensor" in str(e)
