@@ -93,6 +93,9 @@ int check_args(const pat_fwd_args* a) {
   if (a->k_stride[1] * (int64_t)a->page_size >= (int64_t(1) << 29) ||
       a->v_stride[1] * (int64_t)a->page_size >= (int64_t(1) << 29))
     return fail(PAT_ERR_INVALID, "k_cache_paged / v_cache_paged: a block must span less than 1 GiB");
+  // page id x page stride is a 32 x 32 -> 64 bit product in the kernels
+  if (a->k_stride[0] >= (int64_t(1) << 30) || a->v_stride[0] >= (int64_t(1) << 30))
+    return fail(PAT_ERR_INVALID, "k_cache_paged / v_cache_paged: blocks must be less than 2^30 elements apart");
   const void* ptrs[3] = {a->q, a->k, a->v};
   for (int t = 0; t < 3; ++t)
     if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16 != 0)
@@ -145,7 +148,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   int64_t chunk = 0, tall = 0;
   if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
   if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
-  const bool env_tall = tall > 0;
+  const bool env_tall = tall > 0, env_chunk = chunk > 0;
   if (chunk <= 0) {
     // whole multiples of 128 tokens: the 4 waves of a workgroup get the same number of steps,
     // and boxes a little longer than the average do not spill a few tokens into a second chunk
@@ -175,6 +178,15 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     // (a handful of tall boxes stays finely cut: there the tall chain is the critical path)
     if (2 * n > 3 * (int64_t)kResidentWgsPerCU * kNumCUs && n_tall >= kNumCUs)
       tall = std::max<int64_t>(tall, kTallChunkBusy);
+    // Tall workgroups start first and stay for most of the launch. When they take more than a
+    // third of the resident slots, the short boxes' chunk is sized for the slots that are left
+    // (at least one per CU) instead of for two per CU: short workgroups that have to queue behind
+    // the tall ones start late and make the tail.
+    else if (!env_chunk && n_tall > kNumCUs) {
+      const int64_t slots = std::max<int64_t>(kNumCUs, (int64_t)kResidentWgsPerCU * kNumCUs - n_tall);
+      const int64_t c = std::min<int64_t>(kMaxChunk, ceil_div64(ceil_div64(work, slots), 128) * 128);
+      chunk = std::max(chunk, c);
+    }
   }
   g->chunk = (int)std::min(round_unit(chunk), cap);
   g->tall_chunk = (int)std::min(round_unit(tall), cap);

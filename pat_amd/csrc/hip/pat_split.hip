@@ -340,14 +340,29 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       koff[i] = (unsigned)((tok_in[i] & 15) * kss) + col;
       voff[i] = (unsigned)((tok_in[i] & 15) * vss) + col;
     }
+    // Steps are fetched in order, so the half a wave reads next is tracked on the scalar unit
+    // (page of the chunk, 16-token slot in the page, byte offset of the slot) instead of being
+    // derived from the step number every time: a few scalar adds per half. Page strides are
+    // below 4 GiB (checked on the host): page id x stride is one 32 x 32 -> 64 bit multiply.
+    int f_page = 0, f_slot = 0;
+    unsigned f_koff = 0, f_voff = 0;
+    const unsigned ksp32 = (unsigned)ksp, vsp32 = (unsigned)vsp, k16 = (unsigned)(16 * kss), v16 = (unsigned)(16 * vss);
+    auto next_half = [&]() {
+      ++f_slot; f_koff += k16; f_voff += v16;
+      if (f_slot == hpp) { f_slot = 0; f_koff = 0; f_voff = 0; ++f_page; }
+    };
+    // D = 64: one load per step and thread, waves 2 and 3 read the step's second half
+    if (NP == 1 && __builtin_amdgcn_readfirstlane(wave >> 1)) next_half();
     auto fetch = [&](int st, u32x4 (&kd)[NP], u32x4 (&vd)[NP]) {
       if ((st + 1) * kStepTokens <= ntok) {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
-          const int h = __builtin_amdgcn_readfirstlane(st * 2 + (tok_in[i] >> 4));   // uniform over the wave
-          kd[i] = *(const u32x4*)(half_base(kbase, ksp, kss, h) + koff[i]);
-          vd[i] = *(const u32x4*)(half_base(vbase, vsp, vss, h) + voff[i]);
+          const unsigned pg = (unsigned)__builtin_amdgcn_readlane(f_page < 64 ? pg0 : pg1, f_page & 63);
+          kd[i] = *(const u32x4*)(kbase + ((uint64_t)pg * ksp32 + f_koff) + koff[i]);
+          vd[i] = *(const u32x4*)(vbase + ((uint64_t)pg * vsp32 + f_voff) + voff[i]);
+          next_half();
         }
+        if (NP == 1) next_half();
       } else {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {

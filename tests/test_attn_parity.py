@@ -349,6 +349,43 @@ def test_oblivious_plan_same_result_and_linearity():
     assert (out3.float() - 2 * out.float()).abs().max().item() <= 3.2e-2
 
 
+@pytest.mark.parametrize("scale", [-0.1, 0.0, 0.6, 1e-3])
+def test_softmax_scale_sign_zero_and_spread(scale):
+    # the kernel folds the scale's sign into Q and keeps a lazily updated reference maximum: a
+    # negative scale, scale 0 (uniform attention) and a large one (scores spread over +-80, so the
+    # reference maximum has to move many times) must all match the oracle
+    print(f"[case] c3-shaped batch, softmax_scale {scale}", flush=True)
+    dev = _device()
+    w = workloads.make("c2", seed=5)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, scale, out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, w.seq_lens, scale)
+    _assert_close(f"scale {scale}", out, lse, ref_out, ref_lse, w.dtype)
+
+
+def test_reference_maximum_moves_with_sorted_keys():
+    # keys ordered so that every step's scores exceed the previous step's by far more than the
+    # slack of the lazily updated maximum (and then fall again): rescaling on every step of both
+    # the tall and the short path
+    print("[case] sorted keys: growing maxima", flush=True)
+    dev = _device()
+    w = workloads.make("c2", seed=6)
+    q, k, v = w.tensors(dev)
+    q = torch.ones_like(q)
+    ramp = torch.linspace(-3.0, 3.0, k.shape[0] * k.shape[1], device=dev).view(k.shape[0], k.shape[1], 1, 1)
+    k = (ramp * torch.ones_like(k)).to(k.dtype)     # q.k = 128 * ramp, different per page and slot
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("sorted keys", out, lse, ref_out, ref_lse, w.dtype)
+
+
 def test_validation_errors_on_gpu_tensors():
     dev = _device()
     w = workloads.make("c1")
