@@ -351,10 +351,10 @@ def test_oblivious_plan_same_result_and_linearity():
 
 @pytest.mark.parametrize("scale", [-0.1, 0.0, 0.6, 1e-3])
 def test_softmax_scale_sign_zero_and_spread(scale):
-    # the kernel folds the scale's sign into Q and keeps a lazily updated reference maximum: a
-    # negative scale, scale 0 (uniform attention) and a large one (scores spread over +-80, so the
-    # reference maximum has to move many times) must all match the oracle
-    print(f"[case] c3-shaped batch, softmax_scale {scale}", flush=True)
+    # a negative scale, scale 0 (uniform attention), a large one (scores spread over +-80, so the
+    # running maximum moves many times and most probabilities underflow) and a tiny one must all
+    # match the oracle
+    print(f"[case] c2-shaped batch, softmax_scale {scale}", flush=True)
     dev = _device()
     w = workloads.make("c2", seed=5)
     q, k, v = w.tensors(dev)
@@ -371,9 +371,9 @@ def test_softmax_scale_sign_zero_and_spread(scale):
 
 
 def test_reference_maximum_moves_with_sorted_keys():
-    # keys ordered so that every step's scores exceed the previous step's by far more than the
-    # slack of the lazily updated maximum (and then fall again): rescaling on every step of both
-    # the tall and the short path
+    # keys ordered so that the scores of a request grow from page to page by large amounts (and
+    # fall again where its pages go back in the pool): the accumulator is rescaled on most steps
+    # of both the tall and the short path
     print("[case] sorted keys: growing maxima", flush=True)
     dev = _device()
     w = workloads.make("c2", seed=6)
