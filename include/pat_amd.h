@@ -176,7 +176,9 @@ typedef struct pat_fwd_bucket {
 
 /* Mirrors the arguments of pat_mha_fwd_kvcache (csrc/api.h:110-127).
  * Strides are in ELEMENTS (as csrc/api.h:43); the last dimension of q, k, v, out
- * must be contiguous. Unlike the reference, V may have strides of its own. */
+ * must be contiguous. Unlike the reference, V may have strides of its own.
+ * K/V: one block spans less than 2^29 elements (stride[1] * page_size) and blocks
+ * are less than 2^30 elements apart (stride[0]). */
 typedef struct pat_fwd_args {
   int32_t dtype;       /* PAT_DTYPE_F16 | PAT_DTYPE_BF16 (q, k, v, out)      */
   int32_t batch;       /* q.size(0)                                           */
