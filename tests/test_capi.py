@@ -89,6 +89,12 @@ def test_validate_rejects_bad_bucket_and_strides():
     a.k_stride = (C.c_int64 * 3)(16 * 8 * 128 + 4, 8 * 128, 128)
     assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "multiples of 8" in _lib.last_error()
     a = _args()
+    a.v_stride = (C.c_int64 * 3)(1 << 30, 8 * 128, 128)          # blocks 2^30 elements apart
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "2^30 elements apart" in _lib.last_error()
+    a = _args()
+    a.k_stride = (C.c_int64 * 3)(1 << 29, 1 << 25, 128)          # a 16-token block spanning 2^29 elements
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "span less than 1 GiB" in _lib.last_error()
+    a = _args()
     a.buckets[1].max_seqs = 32      # 32 sequences x 4 heads per kv head > 64 rows
     a.buckets[1].q_table_stride = 32
     assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "64 rows" in _lib.last_error()
