@@ -141,7 +141,7 @@ def main() -> None:
     lt = info.launch_tables()   # what prefix_attn_with_kvcache(tree=...) hands to the kernels
     pat_kw = dict(num_split_per_seq=info.num_split_per_seq, query_tables=lt["q_tables"],
                   block_tables=lt["block_tables"], num_seqs_per_CTAs=lt["num_seqs_per_CTAs"],
-                  CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=info.MNWs,
+                  CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=lt["MNWs"],
                   max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                   max_blocks_in_CTA=info.max_blocks_in_CTA)
     pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"])

@@ -51,28 +51,79 @@ class KernelInfo:
         self.max_seqs_in_CTA = 0
         self.max_blocks_in_CTA = 0
         self._launch_cache: dict = {}
-        # Launch copies of the per-bucket tables with every bucket's boxes ordered longest first
-        # (what the kernels are given; the tables above keep the scheduler's order). Workgroups
-        # start in launch order and are dealt round-robin to the CUs, so this order gives every
-        # CU a similar mix and keeps long boxes from starting last.
+        # Launch copies of the per-bucket tables (what the kernels are given; the tables above keep
+        # the scheduler's order): every bucket's boxes longest first, and a bucket whose few widest
+        # boxes are more than twice as long as the rest split in two, so that the kernels do not
+        # reserve workgroups for every box's KV up to the widest one's length. Workgroups start
+        # in launch order and are dealt round-robin to the CUs, so longest-first gives every CU a
+        # similar mix and keeps long boxes from starting last.
         self._launch_tables: Optional[dict] = None
-        self._launch_order: List[torch.Tensor] = []   # per bucket: launch row -> scheduler row
+        self._launch_order: List[torch.Tensor] = []   # per bucket: sorted position -> scheduler row
+        # per bucket: (launch bucket, first sorted position, end) of each part it was split into
+        self._launch_parts: List[List[tuple]] = []
+        self._block_lens: List[np.ndarray] = []       # per bucket and box: block ids in its block_table row
 
     _PER_BOX = ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "slot_tables")
+    _MAX_LAUNCH_BUCKETS = 12      # what one launch of the C ABI takes
+    _GROWTH_BLOCKS = 8
 
     def _sort_for_launch(self) -> None:
+        """Builds the launch copies from the (host) plan tensors."""
         self._launch_order = [torch.argsort(kv, descending=True, stable=True) for kv in self.kv_in_CTAs]
-        self._launch_tables = {
-            name: [t[order].contiguous() for t, order in zip(getattr(self, name), self._launch_order)]
-            for name in self._PER_BOX if getattr(self, name)}
+        names = [name for name in self._PER_BOX if getattr(self, name)]
+        tables = {name: [] for name in names}
+        tables["MNWs"] = []
+        self._launch_parts = []
+        spare = self._MAX_LAUNCH_BUCKETS - len(self.MNWs)
+        for b, order in enumerate(self._launch_order):
+            kv = self.kv_in_CTAs[b][order].numpy()
+            n = len(kv)
+            cuts = [0, n]
+            # a wide head: at most a quarter of the boxes, each more than twice as long as any other
+            if spare > 0 and n >= 4 and b < len(self._block_lens):
+                k = int((kv > kv[0] // 2).sum())
+                if 0 < k <= n // 4:
+                    cuts = [0, k, n]
+                    spare -= 1
+            parts = []
+            for lo, hi in zip(cuts[:-1], cuts[1:]):
+                rows = order[lo:hi]
+                parts.append((len(tables["MNWs"]), lo, hi))
+                tables["MNWs"].append(list(self.MNWs[b]))
+                for name in names:
+                    t = getattr(self, name)[b][rows]
+                    if name == "block_tables" and lo > 0:
+                        # the narrow part: as wide as its widest box, plus room for its boxes to
+                        # grow by a few blocks in place between the steps of multi-step decoding
+                        t = t[:, :max(1, int(self._block_lens[b][rows.numpy()].max()) + self._GROWTH_BLOCKS)]
+                    tables[name].append(t.contiguous())
+            self._launch_parts.append(parts)
+        self._launch_tables = tables
         self._launch_cache.clear()
 
     def launch_tables(self) -> dict:
-        """The per-bucket tables as the kernels get them (longest box first); the scheduler-order
-        tables when no launch copies exist."""
+        """The per-bucket tables as the kernels get them (see `_launch_tables`), with the tile
+        labels of the launch buckets under "MNWs"; the scheduler-order tables when no launch
+        copies exist."""
         if self._launch_tables is not None:
             return self._launch_tables
-        return {name: getattr(self, name) for name in self._PER_BOX}
+        out = {name: getattr(self, name) for name in self._PER_BOX}
+        out["MNWs"] = self.MNWs
+        return out
+
+    def launch_position(self, b: int):
+        """For the boxes of scheduler bucket `b`, in scheduler order: (launch bucket, row in it) as two
+        numpy arrays."""
+        order = self._launch_order[b].cpu().numpy()
+        pos = np.empty(len(order), dtype=np.int64)
+        pos[order] = np.arange(len(order))
+        bucket = np.empty(len(order), dtype=np.int64)
+        row = np.empty(len(order), dtype=np.int64)
+        for lb, lo, hi in self._launch_parts[b]:
+            inside = (pos >= lo) & (pos < hi)
+            bucket[inside] = lb
+            row[inside] = pos[inside] - lo
+        return bucket, row
 
     def to_gpu(self, device: Union[torch.device, str]) -> None:
         """Copies every plan tensor to `device` (asynchronously where the source is pinned)."""
@@ -89,7 +140,8 @@ class KernelInfo:
         self.slot_tables = [move(t) for t in self.slot_tables]
         self.num_split_per_seq = move(self.num_split_per_seq)
         if self._launch_tables is not None:
-            self._launch_tables = {name: [move(t) for t in ts] for name, ts in self._launch_tables.items()}
+            self._launch_tables = {name: (ts if name == "MNWs" else [move(t) for t in ts])
+                                   for name, ts in self._launch_tables.items()}
             self._launch_order = [move(t) for t in self._launch_order]
         self._launch_cache.clear()
 
@@ -114,6 +166,7 @@ class KernelInfo:
             ki.CTA_ranks.append(vec(bk.rank))
             ki.kv_in_CTAs.append(vec(bk.kv))
             ki.slot_tables.append(mat(bk.q_slot, ws))
+            ki._block_lens.append(np.ctypeslib.as_array(bk.block_len, shape=(n,)).copy() if n else np.zeros(0, np.int32))
         ki.num_split_per_seq = torch.from_numpy(
             np.ctypeslib.as_array(view.num_split_per_seq, shape=(view.batch,)).copy())
         ki.max_split_per_seq = view.max_split_per_seq
@@ -344,7 +397,7 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                 lt = info.launch_tables()
                 L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, lt["q_tables"],
                              lt["block_tables"], lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"],
-                             info.MNWs, info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                             lt["MNWs"], info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
                              vals["softmax_scale"], out, lse, lt.get("slot_tables"))
                 if len(info._launch_cache) >= 256:
                     info._launch_cache.clear()

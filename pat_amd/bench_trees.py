@@ -66,7 +66,7 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
     lt = info.launch_tables()   # what prefix_attn_with_kvcache(tree=...) hands to the kernels
     aware = dict(num_split_per_seq=info.num_split_per_seq, query_tables=lt["q_tables"], block_tables=lt["block_tables"],
                  num_seqs_per_CTAs=lt["num_seqs_per_CTAs"], CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"],
-                 MNW=info.MNWs, max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
+                 MNW=lt["MNWs"], max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                  max_blocks_in_CTA=info.max_blocks_in_CTA)
     oblivious = workloads.oblivious_plan(w, dev)
 

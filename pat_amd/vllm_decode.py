@@ -49,7 +49,7 @@ class DecodePlan:
     replans: int = 0                           # times advance_step had to plan afresh
     _tails: Any = None                         # per request (bucket, box) of the item holding its tail
     _tail_kv: Any = None
-    _launch_row: Any = None                    # per bucket: scheduler row -> launch row
+    _launch_row: Any = None                    # per bucket: scheduler row -> (launch bucket, row)
 
     @classmethod
     def from_metadata(cls, meta: Any) -> Optional["DecodePlan"]:
@@ -115,43 +115,52 @@ class DecodePlan:
         if (self._tails[:, 0] < 0).any():
             self._replan(table_cpu)
             return False
-        new_blocks = {}                       # bucket -> ([flat positions], [block ids])
+        new_blocks = {}                       # bucket -> ([box], [column], [block id])
         for s, n_old in enumerate(old):
             if n_old % bs:
                 continue
             b, box = self._tails[s]
-            width = info.block_tables[b].shape[1]
-            pos = -(-int(self._tail_kv[s]) // bs)           # blocks the item holds now
-            if pos >= width:
-                self._replan(table_cpu)
-                return False
-            where, ids = new_blocks.setdefault(int(b), ([], []))
-            where.append(int(box) * width + pos)
+            col = -(-int(self._tail_kv[s]) // bs)           # blocks the item holds now
+            boxes, cols, ids = new_blocks.setdefault(int(b), ([], [], []))
+            boxes.append(int(box))
+            cols.append(col)
             ids.append(int(table_cpu[s, n_old // bs]))
-        self._tail_kv += 1
-        device = info.num_split_per_seq.device
-        # the tables the kernels read (boxes in launch order) and, so that they keep describing the
-        # same plan, the scheduler-order tables
+        # The tables the kernels read are launch copies (boxes in another order, a bucket perhaps
+        # split in two with narrower block tables); the scheduler-order tables are kept in step so
+        # that they go on describing the same plan. (table list, scheduler bucket) -> per table of
+        # the list the rows of the given boxes.
         launch = info.launch_tables()
-        targets = [(info.kv_in_CTAs, info.block_tables, None)]
+        targets = [(info.kv_in_CTAs, info.block_tables, lambda b, boxes: {b: (boxes, np.arange(len(boxes)))})]
         if launch["kv_in_CTAs"] is not info.kv_in_CTAs:
             if self._launch_row is None:
-                self._launch_row = [torch.argsort(order).cpu().numpy() for order in info._launch_order]
-            targets.append((launch["kv_in_CTAs"], launch["block_tables"], self._launch_row))
-        for kvs, tables, row_of in targets:
+                self._launch_row = [info.launch_position(b) for b in range(len(info.MNWs))]
+
+            def in_launch(b, boxes):
+                lb, lr = self._launch_row[b]
+                return {int(t): (lr[boxes[lb[boxes] == t]], np.nonzero(lb[boxes] == t)[0]) for t in np.unique(lb[boxes])}
+            targets.append((launch["kv_in_CTAs"], launch["block_tables"], in_launch))
+        # a block row that is full (in either copy) means a fresh plan
+        for _, tables, place in targets:
+            for b, (boxes, cols, _) in new_blocks.items():
+                for t, (_, which) in place(b, np.asarray(boxes)).items():
+                    if (np.asarray(cols)[which] >= tables[t].shape[1]).any():
+                        self._replan(table_cpu)
+                        return False
+        self._tail_kv += 1
+        device = info.num_split_per_seq.device
+        for kvs, tables, place in targets:
             for b in range(len(info.MNWs)):
-                boxes = self._tails[self._tails[:, 0] == b, 1]
-                width = tables[b].shape[1]
-                if len(boxes):
-                    rows = boxes if row_of is None else row_of[b][boxes]
-                    kvs[b].index_add_(0, torch.as_tensor(rows, device=device),
-                                      torch.ones(len(rows), dtype=torch.int32, device=device))
+                grown = self._tails[self._tails[:, 0] == b, 1]
+                if len(grown):
+                    for t, (rows, _) in place(b, grown).items():
+                        kvs[t].index_add_(0, torch.as_tensor(rows, device=device),
+                                          torch.ones(len(rows), dtype=torch.int32, device=device))
                 if b in new_blocks:
-                    where, ids = new_blocks[b]
-                    if row_of is not None:
-                        where = [int(row_of[b][w // width]) * width + w % width for w in where]
-                    tables[b].view(-1).index_copy_(0, torch.as_tensor(where, device=device),
-                                                   torch.as_tensor(ids, dtype=torch.int32, device=device))
+                    boxes, cols, ids = (np.asarray(x) for x in new_blocks[b])
+                    for t, (rows, which) in place(b, boxes).items():
+                        flat = rows * tables[t].shape[1] + cols[which]
+                        tables[t].view(-1).index_copy_(0, torch.as_tensor(flat, device=device),
+                                                       torch.as_tensor(ids[which], dtype=torch.int32, device=device))
         return True
 
 

@@ -93,12 +93,26 @@ def _table(rows, width):
     return t
 
 
-def test_advance_step_keeps_the_plan_right_on_cpu():
+def _few_long_many_short():
+    """300 unrelated requests, 3 of 640 tokens and 297 of 130..240 (enough of them that the scheduler
+    leaves the long ones whole): a bucket with a wide head, which the launch copies of the plan
+    split in two."""
+    lens = [640, 640, 624] + [130 + (37 * i) % 110 for i in range(296)] + [240]   # 240 = 15 pages: grows at step 1
+    rows, nxt = [], 0
+    for n in lens:
+        nb = -(-n // 16)
+        rows.append(list(range(nxt, nxt + nb)))
+        nxt += nb
+    return workloads.Workload("wide-head", 8, 8, 64, torch.float16, 16, lens, rows, nxt, sum(lens), 0)
+
+
+@pytest.mark.parametrize("case", ["c1", "wide-head"])
+def test_advance_step_keeps_the_plan_right_on_cpu(case):
     """After every in-place advance the plan, executed item by item by the oracle, gives dense
     attention over the grown requests (c1: 8 requests x 288 tokens, so step 1 crosses a page)."""
-    w = workloads.make("c1", seed=5)
+    w = workloads.make("c1", seed=5) if case == "c1" else _few_long_many_short()
     steps = 20
-    spare = list(range(w.num_blocks, w.num_blocks + 64))
+    spare = list(range(w.num_blocks, w.num_blocks + 640))
     width = w.padded_table().shape[1] + 2
     meta = fake_metadata(w, torch.device("cpu"))
     meta.block_tables_cpu = _table(w.rows, width)
@@ -106,8 +120,8 @@ def test_advance_step_keeps_the_plan_right_on_cpu():
     plan = DecodePlan.from_metadata(meta)
     gen = torch.Generator().manual_seed(1)
     q = torch.randn(w.batch, 1, w.heads, w.head_dim, generator=gen)
-    k = torch.randn(w.num_blocks + 64, w.page_size, w.kv_heads, w.head_dim, generator=gen)
-    v = torch.randn(w.num_blocks + 64, w.page_size, w.kv_heads, w.head_dim, generator=gen)
+    k = torch.randn(w.num_blocks + 640, w.page_size, w.kv_heads, w.head_dim, generator=gen)
+    v = torch.randn(w.num_blocks + 640, w.page_size, w.kv_heads, w.head_dim, generator=gen)
     in_place = 0
     for step in range(1, steps + 1):
         rows, lens = _grown(w, step, spare)
@@ -119,10 +133,13 @@ def test_advance_step_keeps_the_plan_right_on_cpu():
                       ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs")}
             listed["num_split_per_seq"] = info.num_split_per_seq.tolist()
             launch = info.launch_tables()       # the kernels' copies (longest box first) grew alike
+            assert (max(len(p) for p in info._launch_parts) == 2) == (case == "wide-head")
             for b, order in enumerate(info._launch_order):
-                assert torch.equal(launch["kv_in_CTAs"][b], info.kv_in_CTAs[b][order])
-                assert torch.equal(launch["block_tables"][b], info.block_tables[b][order])
-                assert (launch["kv_in_CTAs"][b][:-1] >= launch["kv_in_CTAs"][b][1:] - step).all()
+                for lb, lo, hi in info._launch_parts[b]:
+                    lw = launch["block_tables"][lb].shape[1]
+                    assert torch.equal(launch["kv_in_CTAs"][lb], info.kv_in_CTAs[b][order[lo:hi]])
+                    assert torch.equal(launch["block_tables"][lb], info.block_tables[b][order[lo:hi]][:, :lw])
+                    assert (launch["kv_in_CTAs"][lb][:-1] >= launch["kv_in_CTAs"][lb][1:] - step).all()
             out, lse = ao.run_plan_ref(listed, q, k, v)
             ref, ref_lse = ao.paged_attention_ref(q, k, v, rows, lens)
             assert (out - ref).abs().max().item() < 1e-5, step
