@@ -41,6 +41,8 @@ WORKLOAD_TEXT = {
     "c4": "batch 256, forest of 16 roots, depth<=4, 16/16 heads, d64, fp16",
     "c5a": "Llama-3-70B layer shape: batch 32, 16384 shared + U[256,2048], 64/8 heads, d128, bf16",
     "c5b": "batch 32 independent 4096-token contexts, 64/8 heads, d128, bf16",
+    # diagnostic: a launch of 64-row boxes only (profiling the tall-box path)
+    "c5a-prefix": "c5a's 16384-token shared prefix with 16-token suffixes, batch 32, 64/8 heads, d128, bf16",
 }
 
 

@@ -12,6 +12,10 @@ may end inside a page.
        inner U[64,512], leaves U[32,256], 16/16 heads, d 64, fp16
   c5a  32 requests, 16384 shared + U[256,2048] private, 64/8 heads, d 128, bf16
   c5b  32 independent 4096-token requests (no sharing), 64/8 heads, d 128, bf16
+
+A diagnostic beside them (not a benchmark configuration, not in NAMES):
+  c5a-prefix  c5a's shared 16384-token prefix with 16-token private suffixes: a launch made of
+              64-row boxes only, for profiling the tall-box path of the split kernel
 """
 from __future__ import annotations
 
@@ -210,6 +214,8 @@ def make(name: str, seed: int = 0) -> Workload:
         return shared_prefix("c5a", 32, 16384, 256, 2048, 64, 8, 128, bf16, seed)
     if name == "c5b":
         return independent("c5b", 32, 4096, 64, 8, 128, bf16, seed)
+    if name == "c5a-prefix":
+        return shared_prefix("c5a-prefix", 32, 16384, 16, 16, 64, 8, 128, bf16, seed)
     raise KeyError(f"unknown workload {name!r}")
 
 
