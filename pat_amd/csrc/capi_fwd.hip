@@ -26,6 +26,7 @@ constexpr int kTargetWgsPerCU = 2;  // what fits at once: 2 workgroups of 4 wave
 constexpr int kMinChunk = 128;      // tokens
 constexpr int kMaxChunk = 2048;
 constexpr int kTallChunk = 256;
+constexpr int kLongHeadPerWaveChunk = 1024;   // tokens a wave walks alone (long boxes, a kv head per wave)
 constexpr int kTallChunkBusy = 768;          // tall chunk when the launch does not fit on the device at once
 constexpr int kResidentWgsPerCU = 3;
 
@@ -234,6 +235,38 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
       if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= limit) {
         g->bucket_heads_per_wg[i] = kWaves;
         g->total_wgs -= (int64_t)a->buckets[i].num_boxes * (a->kv_heads - a->kv_heads / kWaves);
+      }
+    }
+  }
+  // Long boxes of <= 16 rows in launches far past what the device holds at once: a kv head per
+  // wave there too, on chunks of kLongHeadPerWaveChunk tokens. The 4 waves of a workgroup then read
+  // 4 adjacent heads of the same tokens (1 KB contiguous per token instead of 256 bytes), which
+  // streams ~9 % faster; each wave walks its chunk alone, one step in flight, so this needs enough
+  // queued workgroups to keep every CU's waves busy to the end (a launch that fits at once ends
+  // on its longest chains instead: c3 +11 %, c2 +37 %). PAT_HEAD_PER_WAVE_LONG_WGS overrides the
+  // number of such workgroups a bucket must have (0: always, tuning and tests).
+  if (a->kv_heads % kWaves == 0) {
+    int64_t need = 2 * (int64_t)kResidentWgsPerCU * kNumCUs;
+    if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_WGS")) need = std::atoll(env);
+    bool changed = false;
+    for (int i = 0; i < a->num_buckets; ++i) {
+      const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
+      if (row_tiles(a->buckets[i].mnw[0]) != 1 || g->bucket_heads_per_wg[i] != 1 || tok <= 256) continue;
+      const int64_t c = std::min(round_unit(kLongHeadPerWaveChunk), cap);
+      const int64_t n = ceil_div64(tok, c);
+      if (n > kMaxChunksPerRank) continue;
+      if ((int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need) continue;
+      g->bucket_chunk[i] = (int)c;
+      g->bucket_chunks[i] = (int)n;
+      g->bucket_heads_per_wg[i] = kWaves;
+      changed = true;
+    }
+    if (changed) {
+      g->chunks_per_rank = 1;
+      g->total_wgs = 0;
+      for (int i = 0; i < a->num_buckets; ++i) {
+        g->chunks_per_rank = std::max(g->chunks_per_rank, g->bucket_chunks[i]);
+        g->total_wgs += (int64_t)a->buckets[i].num_boxes * g->bucket_chunks[i] * (a->kv_heads / g->bucket_heads_per_wg[i]);
       }
     }
   }
