@@ -301,6 +301,16 @@ def test_large_ragged_batch_all_launch_modes(heads, dtype):
     out, lse = _run_tree(w, q, k, v)
     ref_out, ref_lse = _oracle(w, q, k, v)
     _assert_close("large ragged", out, lse, ref_out, ref_lse, dtype)
+    # the same batch with a kv head per wave on every bucket of <= 16-row boxes, long ones included
+    # (the geometry a launch with thousands of such workgroups gets by itself)
+    import os
+    os.environ["PAT_HEAD_PER_WAVE_LONG_WGS"] = "0"
+    os.environ["PAT_HEAD_PER_WAVE_TOKENS"] = "256"
+    try:
+        out, lse = _run_tree(w, q, k, v)
+    finally:
+        del os.environ["PAT_HEAD_PER_WAVE_LONG_WGS"], os.environ["PAT_HEAD_PER_WAVE_TOKENS"]
+    _assert_close("large ragged, a kv head per wave", out, lse, ref_out, ref_lse, dtype)
 
 
 def test_strided_views_and_output_in_place():
