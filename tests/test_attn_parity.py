@@ -83,6 +83,35 @@ def test_workload_table_overload(name, dtype):
     _assert_close(f"{name}/{dtype}", out, lse, ref_out, ref_lse, dtype)
 
 
+@pytest.mark.parametrize("kind", ["naive", "compute_model", "sorted"])
+def test_other_plans_of_the_python_scheduler(kind):
+    # plans the kernels see less often: the per-node plan of naive_schedule (no merging, many small
+    # items), the cost-model variant of pack_schedule, and a plan reordered by sort_for_launch
+    print(f"[case] c3 {kind} plan, table form", flush=True)
+    dev = _device()
+    w = workloads.make("c3", seed=3)
+    q, k, v = w.tensors(dev)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    hratio = w.heads // w.kv_heads
+    if kind == "naive":
+        ki = t.naive_schedule(hratio)
+    else:
+        ki = t.pack_schedule(MNWs=None, HRatio=hratio, kvHead=w.kv_heads, use_compute_model=(kind == "compute_model"))
+    if kind == "sorted":
+        ki.sort_for_launch()
+    ki.to_tensor(device=dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                             ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                             ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, None, softmax_lse=lse,
+                             slot_tables=ki.slot_tables or None)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"c3 {kind}", out, lse, ref_out, ref_lse, w.dtype)
+
+
 def test_manual_fixture_partial_pages():
     # the reference's manual fixture (test/test.py:233-239): 33-token requests, partly filled last pages
     print("[case] manual fixture", flush=True)
