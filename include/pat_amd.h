@@ -147,6 +147,51 @@ int pat_tree_pack(pat_tree* tree, const int32_t* mnws, int32_t n_mnws, int32_t h
 /* PrefixTree.naive_schedule(HRatio)           prefix_attn/prefix_tree.py:484-545 */
 int pat_tree_naive_schedule(pat_tree* tree, int32_t hratio);
 
+/* ------------------------------------------------------------------------ *
+ *  The plan as ONE buffer (one host-to-device copy per decode step)         *
+ *  replaces KernelInfo.to_tensor's copy per table, data_class.py:209-254,   *
+ *  and PrefixTreeCPP's tensor aliases, csrc/prefix_tree.h:27-38             *
+ * ------------------------------------------------------------------------ */
+#define PAT_MAX_FLAT_BUCKETS 12
+
+/* One bucket inside the flat buffer: shapes plus the offset of every table, in int32
+ * elements from the start of the buffer. Tables are dense row-major. */
+typedef struct pat_flat_bucket {
+  int32_t mnw[3];
+  int32_t num_boxes;
+  int32_t max_seqs;    /* columns of q_table and q_slot                                  */
+  int32_t max_blocks;  /* columns of block_table                                         */
+  int32_t parent;      /* launch buckets: plan bucket the boxes come from; else own index */
+  int32_t first;       /* launch buckets: position of the first box in the parent's
+                          launch order; plan buckets: 0                                   */
+  int64_t q_table, q_slot, block_table, num_seqs, rank, kv;
+} pat_flat_bucket;
+
+/* Layout of the flat plan. `buckets` is the plan exactly as pat_tree_plan shows it (the
+ * scheduler's order). `launch` holds the copies meant for pat_fwd_launch: every bucket's
+ * boxes longest first (stable), and a bucket in which at most a quarter of the boxes are
+ * more than twice as long as all others split in two (the wide head first), so that the
+ * forward kernels do not reserve work for every box up to the widest one's length; the
+ * second part's block_table is as wide as its widest row plus 8 spare columns (room for
+ * in-place growth between decode steps). launch_order[b] is the offset of plan bucket b's
+ * permutation: entry i = plan row of the box at launch position i. */
+typedef struct pat_flat_plan {
+  int32_t num_buckets;
+  int32_t num_launch_buckets;
+  int32_t batch;
+  int32_t max_split_per_seq, max_seqs_in_box, max_blocks_in_box;
+  int64_t total;               /* int32 elements the buffer needs                        */
+  int64_t num_split_per_seq;   /* offset, [batch]                                        */
+  int64_t launch_order[PAT_MAX_FLAT_BUCKETS];
+  pat_flat_bucket buckets[PAT_MAX_FLAT_BUCKETS];
+  pat_flat_bucket launch[PAT_MAX_FLAT_BUCKETS];
+} pat_flat_plan;
+
+/* Describes the flat form of the current plan in *layout and, when dst is not NULL, writes
+ * it (capacity in int32 elements, at least layout->total). dst may be pinned host memory.
+ * Fails with PAT_ERR_INVALID when the plan has more than PAT_MAX_FLAT_BUCKETS buckets. */
+int pat_tree_flat_plan(const pat_tree* tree, pat_flat_plan* layout, int32_t* dst, int64_t capacity);
+
 /* Borrow the plan built by the last pack / naive_schedule call. */
 int pat_tree_plan(const pat_tree* tree, pat_plan_view* out);
 

@@ -52,6 +52,24 @@ class PlanView(C.Structure):
                 ("max_blocks_in_box", C.c_int32)]
 
 
+class FlatBucket(C.Structure):
+    _fields_ = [("mnw", C.c_int32 * 3), ("num_boxes", C.c_int32), ("max_seqs", C.c_int32),
+                ("max_blocks", C.c_int32), ("parent", C.c_int32), ("first", C.c_int32),
+                ("q_table", C.c_int64), ("q_slot", C.c_int64), ("block_table", C.c_int64),
+                ("num_seqs", C.c_int64), ("rank", C.c_int64), ("kv", C.c_int64)]
+
+
+MAX_FLAT_BUCKETS = 12
+
+
+class FlatPlan(C.Structure):
+    _fields_ = [("num_buckets", C.c_int32), ("num_launch_buckets", C.c_int32), ("batch", C.c_int32),
+                ("max_split_per_seq", C.c_int32), ("max_seqs_in_box", C.c_int32),
+                ("max_blocks_in_box", C.c_int32), ("total", C.c_int64), ("num_split_per_seq", C.c_int64),
+                ("launch_order", C.c_int64 * MAX_FLAT_BUCKETS), ("buckets", FlatBucket * MAX_FLAT_BUCKETS),
+                ("launch", FlatBucket * MAX_FLAT_BUCKETS)]
+
+
 class FwdBucket(C.Structure):
     _fields_ = [("q_table", C.c_void_p), ("block_table", C.c_void_p), ("num_seqs", C.c_void_p),
                 ("rank", C.c_void_p), ("kv", C.c_void_p), ("q_slot", C.c_void_p),
@@ -94,6 +112,7 @@ SYMBOLS = {
                                 C.POINTER(SchedOpts)]),
     "pat_tree_naive_schedule": (C.c_int, [C.c_void_p, C.c_int32]),
     "pat_tree_plan": (C.c_int, [C.c_void_p, C.POINTER(PlanView)]),
+    "pat_tree_flat_plan": (C.c_int, [C.c_void_p, C.POINTER(FlatPlan), C.c_void_p, C.c_int64]),
     "pat_tree_num_nodes": (C.c_int, [C.c_void_p]),
     "pat_tree_node": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(NodeView)]),
     "pat_fwd_validate": (C.c_int, [C.POINTER(FwdArgs)]),

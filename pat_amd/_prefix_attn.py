@@ -62,6 +62,10 @@ class KernelInfo:
         # per bucket: (launch bucket, first sorted position, end) of each part it was split into
         self._launch_parts: List[List[tuple]] = []
         self._block_lens: List[np.ndarray] = []       # per bucket and box: block ids in its block_table row
+        # the whole plan in one int32 buffer (pinned on the host when a GPU is there) of which every
+        # tensor above and every launch copy is a view: one host-to-device copy moves the plan
+        self._flat: Optional[torch.Tensor] = None
+        self._flat_layout: Optional[_lib.FlatPlan] = None
 
     _PER_BOX = ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "slot_tables")
     _MAX_LAUNCH_BUCKETS = 12      # what one launch of the C ABI takes
@@ -128,6 +132,10 @@ class KernelInfo:
     def to_gpu(self, device: Union[torch.device, str]) -> None:
         """Copies every plan tensor to `device` (asynchronously where the source is pinned)."""
         device = torch.device(device)
+        if self._flat is not None:
+            self._flat = self._flat.to(device, non_blocking=True)
+            self._bind(self._flat)
+            return
 
         def move(t: torch.Tensor) -> torch.Tensor:
             return t.to(device, non_blocking=True)
@@ -143,6 +151,61 @@ class KernelInfo:
             self._launch_tables = {name: (ts if name == "MNWs" else [move(t) for t in ts])
                                    for name, ts in self._launch_tables.items()}
             self._launch_order = [move(t) for t in self._launch_order]
+        self._launch_cache.clear()
+
+    @classmethod
+    def _from_flat(cls, native) -> Optional["KernelInfo"]:
+        """The plan of `native` (a `_NativeTree`) as views of one buffer the planner fills, launch
+        copies included; None when the plan has more buckets than the flat form holds."""
+        lib = _lib.load()
+        layout = _lib.FlatPlan()
+        if lib.pat_tree_flat_plan(native._h, C.byref(layout), None, 0) != 0:
+            return None
+        host = torch.empty(max(int(layout.total), 1), dtype=torch.int32, pin_memory=torch.cuda.is_available())
+        _lib.check(lib.pat_tree_flat_plan(native._h, C.byref(layout), C.c_void_p(host.data_ptr()), host.numel()))
+        ki = cls()
+        ki._flat_layout = layout
+        ki._flat = host
+        ki.max_split_per_seq = layout.max_split_per_seq
+        ki.max_seqs_in_CTA = layout.max_seqs_in_box
+        ki.max_blocks_in_CTA = layout.max_blocks_in_box
+        ki._bind(host)
+        return ki
+
+    def _bind(self, flat: torch.Tensor) -> None:
+        """(Re)creates every plan tensor as a view of `flat` (the buffer on the host or its copy on
+        a device)."""
+        lay = self._flat_layout
+
+        def tables(f):
+            n, ws, wb = f.num_boxes, f.max_seqs, f.max_blocks
+            return {"q_tables": flat[f.q_table:f.q_table + n * ws].view(n, ws),
+                    "slot_tables": flat[f.q_slot:f.q_slot + n * ws].view(n, ws),
+                    "block_tables": flat[f.block_table:f.block_table + n * wb].view(n, wb),
+                    "num_seqs_per_CTAs": flat[f.num_seqs:f.num_seqs + n],
+                    "CTA_ranks": flat[f.rank:f.rank + n],
+                    "kv_in_CTAs": flat[f.kv:f.kv + n]}
+
+        self.num_split_per_seq = flat[lay.num_split_per_seq:lay.num_split_per_seq + lay.batch]
+        for name in self._PER_BOX:
+            setattr(self, name, [])
+        self.MNWs, self._launch_order, self._launch_parts = [], [], []
+        for b in range(lay.num_buckets):
+            f = lay.buckets[b]
+            self.MNWs.append([f.mnw[0], f.mnw[1], f.mnw[2]])
+            for name, t in tables(f).items():
+                getattr(self, name).append(t)
+            self._launch_order.append(flat[lay.launch_order[b]:lay.launch_order[b] + f.num_boxes])
+            self._launch_parts.append([])
+        launch = {name: [] for name in self._PER_BOX}
+        launch["MNWs"] = []
+        for i in range(lay.num_launch_buckets):
+            f = lay.launch[i]
+            launch["MNWs"].append([f.mnw[0], f.mnw[1], f.mnw[2]])
+            for name, t in tables(f).items():
+                launch[name].append(t)
+            self._launch_parts[f.parent].append((i, f.first, f.first + f.num_boxes))
+        self._launch_tables = launch
         self._launch_cache.clear()
 
     @classmethod
@@ -212,7 +275,7 @@ class PrefixTreeCPP:
         if MNWs is not None and len(MNWs) == 0:
             MNWs = None  # an empty list selects the default buckets (csrc/prefix_tree.h:189)
         self._native.pack(MNWs, HRatio, kvHead, use_compute_model)
-        self.kernel_info = KernelInfo._from_view(self._native.plan_view())
+        self.kernel_info = KernelInfo._from_flat(self._native) or KernelInfo._from_view(self._native.plan_view())
 
 
 # --------------------------------------------------------------------------------------

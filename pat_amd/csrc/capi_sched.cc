@@ -1,4 +1,5 @@
 // extern "C" surface of the scheduler (declared in include/pat_amd.h).
+#include <algorithm>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -124,6 +125,114 @@ int pat_tree_plan(const pat_tree* tree, pat_plan_view* out) {
   out->max_seqs_in_box = p.max_seqs_in_box;
   out->max_blocks_in_box = p.max_blocks_in_box;
   return PAT_OK;
+}
+
+static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* dst, int64_t capacity) {
+  if (tree == nullptr || layout == nullptr) return pat::fail(PAT_ERR_INVALID, "tree / layout is NULL");
+  const pat::Plan& p = tree->planner->plan();
+  if (!p.valid) return pat::fail(PAT_ERR_INVALID, "no plan: call pat_tree_pack first");
+  const int nb = (int)p.buckets.size();
+  if (nb > PAT_MAX_FLAT_BUCKETS)
+    return pat::fail(PAT_ERR_INVALID, "the flat plan holds at most 12 buckets");
+  constexpr int kGrowthBlocks = 8;
+  std::memset(layout, 0, sizeof(*layout));
+  layout->num_buckets = nb;
+  layout->batch = (int32_t)p.num_split_per_seq.size();
+  layout->max_split_per_seq = p.max_split;
+  layout->max_seqs_in_box = p.max_seqs_in_box;
+  layout->max_blocks_in_box = p.max_blocks_in_box;
+
+  // launch order and parts of every bucket
+  struct Part { int parent, lo, hi, width; };
+  std::vector<std::vector<int32_t>> order((size_t)nb);
+  std::vector<Part> parts;
+  int spare = PAT_MAX_FLAT_BUCKETS - nb;
+  for (int b = 0; b < nb; ++b) {
+    const pat::Bucket& bk = p.buckets[(size_t)b];
+    const int n = (int)bk.kv.size();
+    auto& ord = order[(size_t)b];
+    ord.resize((size_t)n);
+    for (int i = 0; i < n; ++i) ord[(size_t)i] = i;
+    std::stable_sort(ord.begin(), ord.end(), [&](int32_t x, int32_t y) { return bk.kv[(size_t)x] > bk.kv[(size_t)y]; });
+    int cut = 0;
+    if (spare > 0 && n >= 4) {
+      const int32_t widest = bk.kv[(size_t)ord[0]];
+      int k = 0;
+      while (k < n && bk.kv[(size_t)ord[(size_t)k]] > widest / 2) ++k;
+      if (k > 0 && k <= n / 4) { cut = k; --spare; }
+    }
+    if (cut == 0) {
+      parts.push_back({b, 0, n, bk.max_blocks});
+    } else {
+      parts.push_back({b, 0, cut, bk.max_blocks});
+      int32_t longest = 1;
+      for (int i = cut; i < n; ++i) longest = std::max(longest, bk.block_len[(size_t)ord[(size_t)i]]);
+      parts.push_back({b, cut, n, std::min<int32_t>(bk.max_blocks, longest + kGrowthBlocks)});
+    }
+  }
+  layout->num_launch_buckets = (int32_t)parts.size();
+
+  // offsets
+  int64_t at = 0;
+  auto take = [&](int64_t n) { const int64_t o = at; at += n; return o; };
+  layout->num_split_per_seq = take(layout->batch);
+  auto place = [&](pat_flat_bucket& f, const pat::Bucket& bk, int rows, int width, int parent, int first) {
+    std::memcpy(f.mnw, bk.mnw, sizeof(f.mnw));
+    f.num_boxes = rows; f.max_seqs = bk.max_seqs; f.max_blocks = width; f.parent = parent; f.first = first;
+    f.q_table = take((int64_t)rows * bk.max_seqs);
+    f.q_slot = take((int64_t)rows * bk.max_seqs);
+    f.block_table = take((int64_t)rows * width);
+    f.num_seqs = take(rows); f.rank = take(rows); f.kv = take(rows);
+  };
+  for (int b = 0; b < nb; ++b) {
+    const pat::Bucket& bk = p.buckets[(size_t)b];
+    place(layout->buckets[b], bk, (int)bk.kv.size(), bk.max_blocks, b, 0);
+    layout->launch_order[b] = take((int64_t)bk.kv.size());
+  }
+  for (size_t i = 0; i < parts.size(); ++i) {
+    const Part& pt = parts[i];
+    place(layout->launch[i], p.buckets[(size_t)pt.parent], pt.hi - pt.lo, pt.width, pt.parent, pt.lo);
+  }
+  layout->total = at;
+  if (dst == nullptr) return PAT_OK;
+  if (capacity < at) return pat::fail(PAT_ERR_INVALID, "flat plan: buffer too small");
+
+  // contents
+  std::copy(p.num_split_per_seq.begin(), p.num_split_per_seq.end(), dst + layout->num_split_per_seq);
+  auto rows_to = [&](int32_t* out, const std::vector<int32_t>& table, int src_width, int width,
+                     const int32_t* ord, int lo, int hi) {
+    for (int i = lo; i < hi; ++i) {
+      const int32_t* row = table.data() + (size_t)(ord ? ord[i] : i) * (size_t)src_width;
+      std::copy(row, row + width, out + (size_t)(i - lo) * (size_t)width);
+    }
+  };
+  auto vec_to = [&](int32_t* out, const std::vector<int32_t>& v, const int32_t* ord, int lo, int hi) {
+    for (int i = lo; i < hi; ++i) out[i - lo] = v[(size_t)(ord ? ord[i] : i)];
+  };
+  auto fill = [&](const pat_flat_bucket& f, const pat::Bucket& bk, const int32_t* ord, int lo, int hi) {
+    rows_to(dst + f.q_table, bk.q_table, bk.max_seqs, bk.max_seqs, ord, lo, hi);
+    rows_to(dst + f.q_slot, bk.q_slot, bk.max_seqs, bk.max_seqs, ord, lo, hi);
+    rows_to(dst + f.block_table, bk.block_table, bk.max_blocks, f.max_blocks, ord, lo, hi);
+    vec_to(dst + f.num_seqs, bk.num_seqs, ord, lo, hi);
+    vec_to(dst + f.rank, bk.rank, ord, lo, hi);
+    vec_to(dst + f.kv, bk.kv, ord, lo, hi);
+  };
+  for (int b = 0; b < nb; ++b) {
+    const pat::Bucket& bk = p.buckets[(size_t)b];
+    fill(layout->buckets[b], bk, nullptr, 0, (int)bk.kv.size());
+    std::copy(order[(size_t)b].begin(), order[(size_t)b].end(), dst + layout->launch_order[b]);
+  }
+  for (size_t i = 0; i < parts.size(); ++i) {
+    const Part& pt = parts[i];
+    fill(layout->launch[i], p.buckets[(size_t)pt.parent], order[(size_t)pt.parent].data(), pt.lo, pt.hi);
+  }
+  return PAT_OK;
+}
+
+int pat_tree_flat_plan(const pat_tree* tree, pat_flat_plan* layout, int32_t* dst, int64_t capacity) {
+  int rc = PAT_OK;
+  const int thrown = guarded([&] { rc = flat_plan_impl(tree, layout, dst, capacity); });
+  return thrown ? thrown : rc;
 }
 
 int pat_tree_num_nodes(const pat_tree* tree) {

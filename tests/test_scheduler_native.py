@@ -139,3 +139,36 @@ def test_error_mapping():
         c.build_radix_tree([64], torch.zeros(1, 2, dtype=torch.int32))   # needs 4 blocks, table has 2
     with pytest.raises(RuntimeError):
         c.build_radix_tree("nope", torch.zeros(1, 2, dtype=torch.int32))
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5a"])
+def test_flat_plan_equals_the_per_table_view(name):
+    """The one-buffer form of the plan (pat_tree_flat_plan: scheduler-order tables + launch copies,
+    sorted and split by the planner) against the per-table view with the launch copies built in
+    Python: same tables, same launch order, same parts."""
+    from pat_amd import PrefixTreeCPP, workloads
+    from pat_amd._prefix_attn import KernelInfo
+    w = workloads.make(name, seed=1)
+    t = PrefixTreeCPP(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.padded_table())
+    t.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    flat = t.kernel_info
+    assert flat._flat is not None and flat._flat.dim() == 1
+    view = KernelInfo._from_view(t._native.plan_view())
+    assert flat.MNWs == view.MNWs and flat.max_split_per_seq == view.max_split_per_seq
+    assert flat.max_seqs_in_CTA == view.max_seqs_in_CTA and flat.max_blocks_in_CTA == view.max_blocks_in_CTA
+    assert torch.equal(flat.num_split_per_seq, view.num_split_per_seq)
+    names = ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "slot_tables")
+    for key in names:
+        assert all(torch.equal(a, b) for a, b in zip(getattr(flat, key), getattr(view, key))), key
+    fl, vl = flat.launch_tables(), view.launch_tables()
+    assert fl["MNWs"] == vl["MNWs"]
+    for key in names:
+        assert len(fl[key]) == len(vl[key]) and all(torch.equal(a, b) for a, b in zip(fl[key], vl[key])), key
+    assert flat._launch_parts == view._launch_parts
+    assert all(torch.equal(a.long(), b) for a, b in zip(flat._launch_order, view._launch_order))
+    if name == "c4":
+        assert max(len(p) for p in flat._launch_parts) == 2      # a bucket with a wide head
+    # the device copy is one buffer too and its views line up
+    flat.to_gpu("cpu")
+    assert torch.equal(flat.launch_tables()["kv_in_CTAs"][0], vl["kv_in_CTAs"][0])
