@@ -21,6 +21,17 @@ __all__ = ["AsyncTree"]
 _PLANNER = ThreadPoolExecutor(max_workers=1, thread_name_prefix="pat-plan")
 
 
+_COPY_STREAMS: dict = {}
+
+
+def _copy_stream(device: torch.device) -> "torch.cuda.Stream":
+    """The planner thread's upload stream on `device` (default priority), created on first use."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _COPY_STREAMS:
+        _COPY_STREAMS[index] = torch.cuda.Stream(device=index)
+    return _COPY_STREAMS[index]
+
+
 class AsyncTree(PrefixTreeCPP):
     def __init__(self, block_size: int, seq_lens: Union[List[int], torch.Tensor], table: torch.Tensor,
                  MNWs: Optional[List[List[int]]], HRatio: int, kvHead: int, device: torch.device):
@@ -32,7 +43,17 @@ class AsyncTree(PrefixTreeCPP):
             tree = PrefixTreeCPP(block_size)
             tree.build_radix_tree(seq_lens, table)
             tree.pack_schedule(MNWs=MNWs, HRatio=HRatio, kvHead=kvHead)
-            tree.kernel_info.to_gpu(device)
+            dev = torch.device(device)
+            if dev.type == "cuda":
+                # the plan is one pinned buffer: its copy runs on a stream of its own, beside
+                # whatever the model thread has queued, and is complete when this returns, so
+                # the consumer may use any stream
+                stream = _copy_stream(dev)
+                with torch.cuda.stream(stream):
+                    tree.kernel_info.to_gpu(dev)
+                stream.synchronize()
+            else:
+                tree.kernel_info.to_gpu(dev)
             return tree
 
         self._future: Future = _PLANNER.submit(plan)
@@ -42,4 +63,8 @@ class AsyncTree(PrefixTreeCPP):
         """The planned tree; waits for the helper thread and re-raises its exception."""
         if self._tree is None:
             self._tree = self._future.result()
+            flat = self._tree.kernel_info._flat
+            if flat is not None and flat.is_cuda:
+                # allocated on the copy stream, read by kernels of the caller's stream
+                flat.record_stream(torch.cuda.current_stream(flat.device))
         return self._tree

@@ -72,6 +72,30 @@ def test_decode_attention_through_vllm_cache_layout(name):
     assert err <= tol
 
 
+@pytest.mark.gpu
+def test_plan_built_on_the_helper_thread_serves_another_stream():
+    # the helper thread uploads the plan on a stream of its own and returns when the copy is done:
+    # a consumer that runs on a non-default stream right away must see the whole plan
+    print("[case] vLLM decode branch on a side stream", flush=True)
+    dev = torch.device("cuda:0")
+    w = workloads.make("c2", seed=8)
+    q, k, v = w.tensors(dev)
+    kv_cache = torch.stack([k, v])
+    query = q.squeeze(1).contiguous()
+    output = torch.full_like(query, float("nan"))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())        # the inputs were made on the current stream
+    for _ in range(3):                                   # a fresh plan each time, used at once
+        plan = DecodePlan.from_metadata(fake_metadata(w, dev))
+        with torch.cuda.stream(side):
+            decode_attention(query, kv_cache, plan, 1.0 / math.sqrt(w.head_dim), output)
+    side.synchronize()
+    ref, _ = ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, w.seq_lens)
+    err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
+    print(f"[parity] side stream: max|out - ref| = {err:.3e}", flush=True)
+    assert err <= 1.6e-2
+
+
 def _grown(w, steps, spare_blocks):
     """Block table (CPU, padded) and lengths of workload w after `steps` more tokens per request; new
     blocks come from `spare_blocks` in request order."""
