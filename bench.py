@@ -133,7 +133,8 @@ def main() -> None:
             L = _prefix_attn._prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
                                       plan_kw["block_tables"], plan_kw["num_seqs_per_CTAs"], plan_kw["CTA_ranks"],
                                       plan_kw["kv_in_CTAs"], plan_kw["MNW"], plan_kw["max_split_per_seq"],
-                                      plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots)
+                                      plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots,
+                                      plan_kw.get("bucket_flags"))
             launches.append(L)
         ws = torch.empty(max(L.need for L in launches), dtype=torch.uint8, device=dev)
         for L in launches:
@@ -145,7 +146,7 @@ def main() -> None:
                   block_tables=lt["block_tables"], num_seqs_per_CTAs=lt["num_seqs_per_CTAs"],
                   CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=lt["MNWs"],
                   max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
-                  max_blocks_in_CTA=info.max_blocks_in_CTA)
+                  max_blocks_in_CTA=info.max_blocks_in_CTA, bucket_flags=lt.get("flags"))
     pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"])
 
     def step(launches, i):

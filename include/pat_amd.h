@@ -164,6 +164,8 @@ typedef struct pat_flat_bucket {
   int32_t parent;      /* launch buckets: plan bucket the boxes come from; else own index */
   int32_t first;       /* launch buckets: position of the first box in the parent's
                           launch order; plan buckets: 0                                   */
+  int32_t flags;       /* PAT_BUCKET_* hints that hold for the bucket                    */
+  int32_t pad_;
   int64_t q_table, q_slot, block_table, num_seqs, rank, kv;
 } pat_flat_bucket;
 
@@ -217,7 +219,14 @@ typedef struct pat_fwd_bucket {
   int32_t max_seqs;           /* valid columns of q_table                     */
   int32_t max_blocks;         /* valid columns of block_table                 */
   int32_t mnw[3];
+  int32_t flags;              /* PAT_BUCKET_* hints, 0 when nothing is known  */
 } pat_fwd_bucket;
+
+/* Hint: no box of the bucket is shorter than 3/4 of its widest box (the launcher cannot see
+ * lengths, which live in device memory). Long even buckets get one kv head per wave sooner
+ * (contiguous reads across heads; safe only when no workgroup outlasts the others by much).
+ * A wrong hint costs time, never correctness. */
+#define PAT_BUCKET_EVEN 1
 
 /* Mirrors the arguments of pat_mha_fwd_kvcache (csrc/api.h:110-127).
  * Strides are in ELEMENTS (as csrc/api.h:43); the last dimension of q, k, v, out

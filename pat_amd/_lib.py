@@ -55,7 +55,7 @@ class PlanView(C.Structure):
 class FlatBucket(C.Structure):
     _fields_ = [("mnw", C.c_int32 * 3), ("num_boxes", C.c_int32), ("max_seqs", C.c_int32),
                 ("max_blocks", C.c_int32), ("parent", C.c_int32), ("first", C.c_int32),
-                ("q_table", C.c_int64), ("q_slot", C.c_int64), ("block_table", C.c_int64),
+                ("flags", C.c_int32), ("pad_", C.c_int32), ("q_table", C.c_int64), ("q_slot", C.c_int64), ("block_table", C.c_int64),
                 ("num_seqs", C.c_int64), ("rank", C.c_int64), ("kv", C.c_int64)]
 
 
@@ -75,7 +75,10 @@ class FwdBucket(C.Structure):
                 ("rank", C.c_void_p), ("kv", C.c_void_p), ("q_slot", C.c_void_p),
                 ("q_table_stride", C.c_int64), ("block_table_stride", C.c_int64),
                 ("num_boxes", C.c_int32), ("max_seqs", C.c_int32), ("max_blocks", C.c_int32),
-                ("mnw", C.c_int32 * 3)]
+                ("mnw", C.c_int32 * 3), ("flags", C.c_int32)]
+
+
+PAT_BUCKET_EVEN = 1
 
 
 class FwdArgs(C.Structure):

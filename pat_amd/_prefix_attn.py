@@ -148,7 +148,7 @@ class KernelInfo:
         self.slot_tables = [move(t) for t in self.slot_tables]
         self.num_split_per_seq = move(self.num_split_per_seq)
         if self._launch_tables is not None:
-            self._launch_tables = {name: (ts if name == "MNWs" else [move(t) for t in ts])
+            self._launch_tables = {name: (ts if name in ("MNWs", "flags") else [move(t) for t in ts])
                                    for name, ts in self._launch_tables.items()}
             self._launch_order = [move(t) for t in self._launch_order]
         self._launch_cache.clear()
@@ -198,10 +198,11 @@ class KernelInfo:
             self._launch_order.append(flat[lay.launch_order[b]:lay.launch_order[b] + f.num_boxes])
             self._launch_parts.append([])
         launch = {name: [] for name in self._PER_BOX}
-        launch["MNWs"] = []
+        launch["MNWs"], launch["flags"] = [], []
         for i in range(lay.num_launch_buckets):
             f = lay.launch[i]
             launch["MNWs"].append([f.mnw[0], f.mnw[1], f.mnw[2]])
+            launch["flags"].append(int(f.flags))
             for name, t in tables(f).items():
                 launch[name].append(t)
             self._launch_parts[f.parent].append((i, f.first, f.first + f.num_boxes))
@@ -292,7 +293,7 @@ class _Launch:
 
 
 def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MNW, max_split,
-             max_seqs, max_blocks, scale, out, lse, slot_tables=None) -> _Launch:
+             max_seqs, max_blocks, scale, out, lse, slot_tables=None, bucket_flags=None) -> _Launch:
     lib = _lib.load()
     # --- checks that need tensor metadata (csrc/api.h:131-181, :256-277) -----------------
     _check(q.dtype in (torch.float16, torch.bfloat16), "only support fp16 and bf16 data type")
@@ -344,6 +345,7 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
         fb.block_table_stride = bt.stride(0) if ctas > 1 else max(bt.shape[1], 1)
         fb.num_boxes, fb.max_seqs, fb.max_blocks = ctas, qt.shape[1], bt.shape[1]
         fb.mnw[0], fb.mnw[1], fb.mnw[2] = int(MNW[i][0]), int(MNW[i][1]), int(MNW[i][2])
+        fb.flags = int(bucket_flags[i]) if bucket_flags else 0
 
     a = _lib.FwdArgs()
     a.dtype = _lib.PAT_DTYPE_BF16 if q.dtype == torch.bfloat16 else _lib.PAT_DTYPE_F16
@@ -390,7 +392,7 @@ def _run(L: _Launch, device: torch.device) -> None:
 _TABLE_LAUNCHES: dict = {}
 
 
-def _table_key(q, k, v, out, lse, vals, slots):
+def _table_key(q, k, v, out, lse, vals, slots, flags=None):
     """Identity of a table-form call: every tensor's address and layout plus the scalars. None when
     the arguments are not what a well-formed call passes (the full checks then raise)."""
     try:
@@ -403,7 +405,8 @@ def _table_key(q, k, v, out, lse, vals, slots):
         return (ident(q), ident(k), ident(v), ident(out), q.dtype, None if lse is None else ident(lse),
                 small(vals["num_split_per_seq"]), lists, tuple(tuple(m) for m in vals["MNW"]),
                 int(vals["max_split_per_seq"]), int(vals["max_seqs_in_CTA"]), int(vals["max_blocks_in_CTA"]),
-                float(vals["softmax_scale"]), None if not slots else tuple(small(t) for t in slots))
+                float(vals["softmax_scale"]), None if not slots else tuple(small(t) for t in slots),
+                None if not flags else tuple(int(f) for f in flags))
     except (AttributeError, TypeError, ValueError):
         return None
 
@@ -420,10 +423,13 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
     natural-log LSE, which the reference computes but does not return. The table form also
     accepts `slot_tables` (`KernelInfo.slot_tables`): with it, partial results are filed by each
     box's ordinal within its sequence instead of by CTA_rank, which stays correct on batches
-    where the reference scheduler hands the same rank to two boxes of one sequence.
+    where the reference scheduler hands the same rank to two boxes of one sequence; and
+    `bucket_flags` (one int per bucket, `PAT_BUCKET_EVEN` = 1 when no box of the bucket is shorter
+    than 3/4 of its widest: a hint for the launch geometry, never needed for correctness).
     """
     lse = kw.pop("softmax_lse", None)
     slots = kw.pop("slot_tables", None)
+    flags = kw.pop("bucket_flags", None)
     tree_names = ("tree", "softmax_scale", "out")
     table_names = ("num_split_per_seq", "query_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks",
                    "kv_in_CTAs", "MNW", "max_split_per_seq", "max_seqs_in_CTA", "max_blocks_in_CTA",
@@ -461,7 +467,7 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                 L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, lt["q_tables"],
                              lt["block_tables"], lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"],
                              lt["MNWs"], info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
-                             vals["softmax_scale"], out, lse, lt.get("slot_tables"))
+                             vals["softmax_scale"], out, lse, lt.get("slot_tables"), lt.get("flags"))
                 if len(info._launch_cache) >= 256:
                     info._launch_cache.clear()
                 info._launch_cache[key] = L
@@ -470,13 +476,13 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
             # with the same plan, and building the argument block costs more than the kernels of a
             # small batch take. The key holds what the block was built from (addresses and
             # layouts); the tensors' contents are read by the kernels at every call.
-            key = _table_key(q, k_cache_paged, v_cache_paged, out, lse, vals, slots)
+            key = _table_key(q, k_cache_paged, v_cache_paged, out, lse, vals, slots, flags)
             L = _TABLE_LAUNCHES.get(key) if key is not None else None
             if L is None:
                 L = _prepare(q, k_cache_paged, v_cache_paged, vals["num_split_per_seq"], vals["query_tables"],
                              vals["block_tables"], vals["num_seqs_per_CTAs"], vals["CTA_ranks"], vals["kv_in_CTAs"],
                              vals["MNW"], vals["max_split_per_seq"], vals["max_seqs_in_CTA"],
-                             vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse, slots)
+                             vals["max_blocks_in_CTA"], vals["softmax_scale"], out, lse, slots, flags)
                 if key is not None:
                     if len(_TABLE_LAUNCHES) >= 64:
                         _TABLE_LAUNCHES.clear()

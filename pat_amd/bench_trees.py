@@ -67,14 +67,15 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
     aware = dict(num_split_per_seq=info.num_split_per_seq, query_tables=lt["q_tables"], block_tables=lt["block_tables"],
                  num_seqs_per_CTAs=lt["num_seqs_per_CTAs"], CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"],
                  MNW=lt["MNWs"], max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
-                 max_blocks_in_CTA=info.max_blocks_in_CTA)
+                 max_blocks_in_CTA=info.max_blocks_in_CTA, bucket_flags=lt.get("flags"))
     oblivious = workloads.oblivious_plan(w, dev)
 
     def launches(plan, slots):
         made = [_prefix_attn._prepare(q, ks[i], vs[i], plan["num_split_per_seq"], plan["query_tables"],
                                       plan["block_tables"], plan["num_seqs_per_CTAs"], plan["CTA_ranks"],
                                       plan["kv_in_CTAs"], plan["MNW"], plan["max_split_per_seq"],
-                                      plan["max_seqs_in_CTA"], plan["max_blocks_in_CTA"], scale, out, None, slots)
+                                      plan["max_seqs_in_CTA"], plan["max_blocks_in_CTA"], scale, out, None, slots,
+                                      plan.get("bucket_flags"))
                 for i in range(len(ks))]
         ws = torch.empty(made[0].need, dtype=torch.uint8, device=dev)
         for m in made:

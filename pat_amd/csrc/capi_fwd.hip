@@ -247,7 +247,8 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   // number of such workgroups a bucket must have (0: always, tuning and tests).
   if (a->kv_heads % kWaves == 0) {
     int64_t need = 2 * (int64_t)kResidentWgsPerCU * kNumCUs;
-    if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_WGS")) need = std::atoll(env);
+    bool forced = false;
+    if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_WGS")) { need = std::atoll(env); forced = true; }
     bool changed = false;
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
@@ -255,7 +256,9 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
       const int64_t c = std::min(round_unit(kLongHeadPerWaveChunk), cap);
       const int64_t n = ceil_div64(tok, c);
       if (n > kMaxChunksPerRank) continue;
-      if ((int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need) continue;
+      // an even bucket (caller's hint) has no stragglers: one such workgroup per CU is enough
+      const int64_t need_i = (a->buckets[i].flags & PAT_BUCKET_EVEN) && !forced ? std::min<int64_t>(need, kNumCUs) : need;
+      if ((int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need_i) continue;
       g->bucket_chunk[i] = (int)c;
       g->bucket_chunks[i] = (int)n;
       g->bucket_heads_per_wg[i] = kWaves;

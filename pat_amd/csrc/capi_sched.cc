@@ -1,5 +1,7 @@
 // extern "C" surface of the scheduler (declared in include/pat_amd.h).
 #include <algorithm>
+#include <climits>
+#include <cstdint>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -179,6 +181,7 @@ static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* 
   auto place = [&](pat_flat_bucket& f, const pat::Bucket& bk, int rows, int width, int parent, int first) {
     std::memcpy(f.mnw, bk.mnw, sizeof(f.mnw));
     f.num_boxes = rows; f.max_seqs = bk.max_seqs; f.max_blocks = width; f.parent = parent; f.first = first;
+    f.flags = 0;
     f.q_table = take((int64_t)rows * bk.max_seqs);
     f.q_slot = take((int64_t)rows * bk.max_seqs);
     f.block_table = take((int64_t)rows * width);
@@ -193,6 +196,19 @@ static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* 
     const Part& pt = parts[i];
     place(layout->launch[i], p.buckets[(size_t)pt.parent], pt.hi - pt.lo, pt.width, pt.parent, pt.lo);
   }
+  // hints: a bucket is even when no box is shorter than 3/4 of its widest one
+  auto even = [&](const pat::Bucket& bk, const int32_t* ord, int lo, int hi) {
+    int32_t widest = 0, shortest = INT32_MAX;
+    for (int i = lo; i < hi; ++i) {
+      const int32_t t = bk.kv[(size_t)(ord ? ord[i] : i)];
+      widest = std::max(widest, t); shortest = std::min(shortest, t);
+    }
+    return hi > lo && (int64_t)shortest * 4 >= (int64_t)widest * 3 ? PAT_BUCKET_EVEN : 0;
+  };
+  for (int b = 0; b < nb; ++b)
+    layout->buckets[b].flags = even(p.buckets[(size_t)b], nullptr, 0, (int)p.buckets[(size_t)b].kv.size());
+  for (size_t i = 0; i < parts.size(); ++i)
+    layout->launch[i].flags = even(p.buckets[(size_t)parts[i].parent], order[(size_t)parts[i].parent].data(), parts[i].lo, parts[i].hi);
   layout->total = at;
   if (dst == nullptr) return PAT_OK;
   if (capacity < at) return pat::fail(PAT_ERR_INVALID, "flat plan: buffer too small");

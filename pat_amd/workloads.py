@@ -239,4 +239,9 @@ def oblivious_plan(w: Workload, device) -> dict:
         kv_in_CTAs=[torch.tensor(w.seq_lens, dtype=torch.int32, device=device)],
         MNW=[label],
         max_split_per_seq=1, max_seqs_in_CTA=1, max_blocks_in_CTA=max(len(r) for r in w.rows),
+        # the hint the prefix-aware plan's launch copies carry (PAT_BUCKET_EVEN), where it serves
+        # this plan too: requests of even length that share nothing (with shared pages the rule it
+        # switches on makes this plan slower, c2: 64 -> 73 us, and the comparison should be against
+        # the faster form)
+        bucket_flags=[1 if 4 * min(w.seq_lens) >= 3 * max(w.seq_lens) and w.unique_tokens >= w.total_tokens else 0],
     )
