@@ -172,3 +172,19 @@ def test_flat_plan_equals_the_per_table_view(name):
     # the device copy is one buffer too and its views line up
     flat.to_gpu("cpu")
     assert torch.equal(flat.launch_tables()["kv_in_CTAs"][0], vl["kv_in_CTAs"][0])
+
+
+def test_flat_plan_marks_even_buckets():
+    from pat_amd import PrefixTreeCPP, workloads
+    flags = {}
+    for name in ("c5b", "c3"):
+        w = workloads.make(name, seed=0)
+        t = PrefixTreeCPP(w.page_size)
+        t.build_radix_tree(w.seq_lens, w.padded_table())
+        t.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+        lt = t.kernel_info.launch_tables()
+        flags[name] = lt["flags"]
+        for f, kv in zip(lt["flags"], lt["kv_in_CTAs"]):
+            assert f == (1 if 4 * int(kv.min()) >= 3 * int(kv.max()) else 0)
+    assert flags["c5b"] == [1]          # 32 requests of 4096 tokens
+    assert flags["c3"][-1] == 0         # leaves of 128..1024 tokens
