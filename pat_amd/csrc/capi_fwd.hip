@@ -253,8 +253,10 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
       if (row_tiles(a->buckets[i].mnw[0]) != 1 || g->bucket_heads_per_wg[i] != 1 || tok <= 256) continue;
-      const int64_t c = std::min(round_unit(kLongHeadPerWaveChunk), cap);
-      const int64_t n = ceil_div64(tok, c);
+      int64_t want = kLongHeadPerWaveChunk;
+      if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_TOKENS")) want = std::max<int64_t>(32, std::atoll(env));
+      const int64_t n = ceil_div64(tok, std::min(round_unit(want), cap));
+      const int64_t c = std::min(round_unit(ceil_div64(tok, n)), cap);   // n even pieces of the widest box
       if (n > kMaxChunksPerRank) continue;
       // an even bucket (caller's hint) has no stragglers: one such workgroup per CU is enough
       const int64_t need_i = (a->buckets[i].flags & PAT_BUCKET_EVEN) && !forced ? std::min<int64_t>(need, kNumCUs) : need;
