@@ -290,6 +290,36 @@ typedef struct pat_fwd_geometry {
 } pat_fwd_geometry;
 int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out);
 
+/* ------------------------------------------------------------------------ *
+ *  Prefix-oblivious paged decode: the comparator of the benchmarks          *
+ *  (benchmark/benchmark_kernel.py runs FlashAttention / FlashInfer decode   *
+ *  beside PAT, :270-330; here the same two kernels run the plan that        *
+ *  block_scheduler.pack_without_prefix describes, prefix_attn/              *
+ *  block_scheduler.py:155-202: one work item per request over its own block *
+ *  row, split along KV by the launch geometry)                              *
+ * ------------------------------------------------------------------------ */
+typedef struct pat_baseline_args {
+  int32_t dtype, batch, heads, kv_heads, head_dim, page_size, num_pages;
+  int32_t max_blocks;            /* columns of block_table in use                 */
+  const void* q;                 /* [batch, 1, heads, head_dim]                   */
+  const void* k;                 /* [num_pages, page_size, kv_heads, head_dim]    */
+  const void* v;
+  void* out;                     /* like q                                        */
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];   /* as pat_fwd_args */
+  const int32_t* block_table;    /* device [batch, block_table_stride]            */
+  int64_t block_table_stride;
+  const int32_t* seq_lens;       /* device [batch], tokens                        */
+  float softmax_scale;
+  int32_t flags;                 /* PAT_BUCKET_* hints for the one bucket         */
+  float* lse_out;                /* optional device [batch, heads]                */
+  void* workspace;               /* device, 256-byte aligned                      */
+  size_t workspace_bytes;
+} pat_baseline_args;
+
+int pat_paged_decode_baseline_workspace_bytes(const pat_baseline_args* args, size_t* bytes);
+/* Enqueues a small table-fill kernel, the split kernel and the merge kernel on the stream. */
+int pat_paged_decode_baseline_launch(const pat_baseline_args* args, void* hip_stream);
+
 /* Device self-test (no counterpart in the reference): runs a one-wave kernel on `hip_stream` that
  * checks the lane-swap reductions and the transposed LDS read against their definitions - the
  * instruction-level facts the split kernel is built on - and stores the number of mismatches in

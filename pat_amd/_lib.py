@@ -81,6 +81,17 @@ class FwdBucket(C.Structure):
 PAT_BUCKET_EVEN = 1
 
 
+class BaselineArgs(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("batch", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32),
+                ("head_dim", C.c_int32), ("page_size", C.c_int32), ("num_pages", C.c_int32),
+                ("max_blocks", C.c_int32), ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p),
+                ("out", C.c_void_p), ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3),
+                ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3), ("block_table", C.c_void_p),
+                ("block_table_stride", C.c_int64), ("seq_lens", C.c_void_p), ("softmax_scale", C.c_float),
+                ("flags", C.c_int32), ("lse_out", C.c_void_p), ("workspace", C.c_void_p),
+                ("workspace_bytes", C.c_size_t)]
+
+
 class FwdArgs(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("batch", C.c_int32), ("seqlen_q", C.c_int32),
                 ("heads", C.c_int32), ("kv_heads", C.c_int32), ("head_dim", C.c_int32),
@@ -121,6 +132,8 @@ SYMBOLS = {
     "pat_fwd_validate": (C.c_int, [C.POINTER(FwdArgs)]),
     "pat_fwd_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_launch": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "pat_paged_decode_baseline_workspace_bytes": (C.c_int, [C.POINTER(BaselineArgs), C.POINTER(C.c_size_t)]),
+    "pat_paged_decode_baseline_launch": (C.c_int, [C.POINTER(BaselineArgs), C.c_void_p]),
     "pat_fwd_geometry_of": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(FwdGeometry)]),
     "pat_selftest_device": (C.c_int, [C.c_void_p, C.POINTER(C.c_int32)]),
 }

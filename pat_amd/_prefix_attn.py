@@ -24,7 +24,7 @@ from .prefix_tree import _NativeTree
 
 _current_device = getattr(torch._C, "_cuda_getDevice", torch.cuda.current_device)
 
-__all__ = ["prefix_attn_with_kvcache", "PrefixTreeCPP", "KernelInfo"]
+__all__ = ["prefix_attn_with_kvcache", "PrefixTreeCPP", "KernelInfo", "paged_decode_baseline"]
 
 
 def _check(cond: bool, msg: str) -> None:
@@ -488,3 +488,52 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
                         _TABLE_LAUNCHES.clear()
                     _TABLE_LAUNCHES[key] = L
         _run(L, q.device)
+
+
+def paged_decode_baseline(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cache_paged: torch.Tensor,
+                          block_table: torch.Tensor, seq_lens: torch.Tensor, softmax_scale: float,
+                          out: torch.Tensor, softmax_lse: Optional[torch.Tensor] = None,
+                          even_lengths: bool = False) -> None:
+    """Prefix-oblivious paged decode attention, the comparator of the benchmarks (not part of the
+    reference's API): every request is one work item over its own row of `block_table` (device
+    int32 `[batch, max_blocks]`), `seq_lens` (device int32 `[batch]`) tokens long; the same split
+    and merge kernels run it. `even_lengths`: no request is shorter than 3/4 of the longest."""
+    for name, t in (("q", q), ("kcache", k_cache_paged), ("vcache", v_cache_paged), ("block_table", block_table),
+                    ("seq_lens", seq_lens)):
+        _check(isinstance(t, torch.Tensor) and t.is_cuda, f"{name} must be on CUDA")
+    _check(q.dtype in (torch.float16, torch.bfloat16) and k_cache_paged.dtype == q.dtype and v_cache_paged.dtype == q.dtype,
+           "only support fp16 and bf16 data type")
+    _check(q.dim() == 4 and k_cache_paged.dim() == 4 and v_cache_paged.dim() == 4, "q, kcache, vcache must be 4-D")
+    _check(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+           "block_table must be a 2-D int32 tensor with contiguous rows")
+    _check(seq_lens.dtype == torch.int32 and seq_lens.dim() == 1 and seq_lens.is_contiguous(),
+           "seq_lens must be a contiguous 1-D int32 tensor")
+    b, sq, h, d = q.shape
+    _check(sq == 1, "q must have shape (batch_size, 1, n_heads, head_size): decode only")
+    _check(block_table.shape[0] == b and seq_lens.shape[0] == b, "block_table / seq_lens must have one row per request")
+    _check(out.is_cuda and out.dtype == q.dtype and tuple(out.shape) == tuple(q.shape) and out.stride(-1) == 1,
+           "out must be a CUDA tensor with q's shape and dtype and a contiguous last dimension")
+    lib = _lib.load()
+    a = _lib.BaselineArgs()
+    a.dtype = _lib.PAT_DTYPE_BF16 if q.dtype == torch.bfloat16 else _lib.PAT_DTYPE_F16
+    a.batch, a.heads, a.kv_heads, a.head_dim = b, h, k_cache_paged.shape[2], d
+    a.page_size, a.num_pages, a.max_blocks = k_cache_paged.shape[1], k_cache_paged.shape[0], block_table.shape[1]
+    a.q, a.k, a.v, a.out = q.data_ptr(), k_cache_paged.data_ptr(), v_cache_paged.data_ptr(), out.data_ptr()
+    a.q_stride, a.k_stride, a.v_stride, a.o_stride = (_strides3(q), _strides3(k_cache_paged), _strides3(v_cache_paged),
+                                                      _strides3(out))
+    a.block_table, a.block_table_stride = block_table.data_ptr(), block_table.stride(0)
+    a.seq_lens = seq_lens.data_ptr()
+    a.softmax_scale = float(softmax_scale)
+    a.flags = _lib.PAT_BUCKET_EVEN if even_lengths else 0
+    if softmax_lse is not None:
+        _check(softmax_lse.is_cuda and softmax_lse.dtype == torch.float32 and softmax_lse.is_contiguous()
+               and softmax_lse.numel() == b * h, "softmax_lse must be a contiguous CUDA float32 tensor with batch_size * n_heads elements")
+        a.lse_out = softmax_lse.data_ptr()
+    need = C.c_size_t(0)
+    _lib.check(lib.pat_paged_decode_baseline_workspace_bytes(C.byref(a), C.byref(need)))
+    index = q.device.index
+    guard = torch.cuda.device(index) if index != _current_device() else contextlib.nullcontext()
+    with guard:
+        ws = torch.empty(need.value, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+        _lib.check(lib.pat_paged_decode_baseline_launch(C.byref(a), C.c_void_p(_raw_stream(index))))

@@ -411,4 +411,94 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   return PAT_OK;
 }
 
+// ---- prefix-oblivious comparator ------------------------------------------------------------
+namespace {
+// one request per work item: q_table row i = {i}, one sequence each, rank 0, one split
+__global__ void pat_baseline_tables_kernel(int32_t* q_table, int32_t* ones, int32_t* zeros, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) { q_table[i] = i; ones[i] = 1; zeros[i] = 0; }
+}
+
+size_t baseline_tables_bytes(int batch) { return pat::align256((size_t)batch * sizeof(int32_t)) * 3; }
+
+int baseline_fwd_args(const pat_baseline_args* b, pat_fwd_args* a, pat_fwd_bucket* bucket) {
+  if (b == nullptr) return pat::fail(PAT_ERR_INVALID, "args is NULL");
+  if (b->batch <= 0) return pat::fail(PAT_ERR_INVALID, "batch size must be positive");
+  if (b->kv_heads <= 0 || b->heads <= 0 || b->heads % b->kv_heads != 0)
+    return pat::fail(PAT_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
+  if (b->block_table == nullptr || b->seq_lens == nullptr)
+    return pat::fail(PAT_ERR_INVALID, "block_table / seq_lens must be device int32 tensors");
+  if (b->max_blocks <= 0 || b->block_table_stride < b->max_blocks)
+    return pat::fail(PAT_ERR_INVALID, "block_table must have max_blocks > 0 columns within its row stride");
+  std::memset(a, 0, sizeof(*a));
+  std::memset(bucket, 0, sizeof(*bucket));
+  a->dtype = b->dtype; a->batch = b->batch; a->seqlen_q = 1; a->heads = b->heads; a->kv_heads = b->kv_heads;
+  a->head_dim = b->head_dim; a->page_size = b->page_size; a->num_pages = b->num_pages;
+  a->q = b->q; a->k = b->k; a->v = b->v; a->out = b->out; a->lse_out = b->lse_out;
+  for (int i = 0; i < 3; ++i) {
+    a->q_stride[i] = b->q_stride[i]; a->k_stride[i] = b->k_stride[i];
+    a->v_stride[i] = b->v_stride[i]; a->o_stride[i] = b->o_stride[i];
+  }
+  a->max_split_per_seq = 1; a->max_seqs_in_box = 1; a->max_blocks_in_box = b->max_blocks;
+  a->softmax_scale = b->softmax_scale;
+  // the tables the fill kernel writes live at the start of the workspace
+  char* ws = static_cast<char*>(b->workspace);
+  const size_t one = pat::align256((size_t)b->batch * sizeof(int32_t));
+  int32_t* q_table = reinterpret_cast<int32_t*>(ws);
+  int32_t* ones = reinterpret_cast<int32_t*>(ws ? ws + one : nullptr);
+  int32_t* zeros = reinterpret_cast<int32_t*>(ws ? ws + 2 * one : nullptr);
+  // (addresses only have to be non-null for the checks when no workspace is given yet)
+  static int32_t placeholder;
+  bucket->q_table = ws ? q_table : &placeholder;
+  bucket->num_seqs = ws ? ones : &placeholder;
+  bucket->rank = ws ? zeros : &placeholder;
+  bucket->block_table = b->block_table; bucket->kv = b->seq_lens;
+  bucket->q_table_stride = 1; bucket->block_table_stride = b->block_table_stride;
+  bucket->num_boxes = b->batch; bucket->max_seqs = 1; bucket->max_blocks = b->max_blocks;
+  const int rows = b->heads / b->kv_heads;
+  bucket->mnw[0] = rows <= 16 ? 16 : (rows <= 32 ? 32 : 64); bucket->mnw[1] = 128; bucket->mnw[2] = 1;
+  bucket->flags = b->flags;
+  a->num_split_per_seq = ws ? ones : &placeholder;
+  a->num_buckets = 1; a->buckets = bucket;
+  if (ws != nullptr) {
+    a->workspace = ws + baseline_tables_bytes(b->batch);
+    a->workspace_bytes = b->workspace_bytes > baseline_tables_bytes(b->batch) ? b->workspace_bytes - baseline_tables_bytes(b->batch) : 0;
+  }
+  return PAT_OK;
+}
+}  // namespace
+
+int pat_paged_decode_baseline_workspace_bytes(const pat_baseline_args* args, size_t* bytes) {
+  if (bytes == nullptr) return pat::fail(PAT_ERR_INVALID, "bytes is NULL");
+  pat_fwd_args a; pat_fwd_bucket bucket;
+  pat_baseline_args probe;
+  if (args == nullptr) return pat::fail(PAT_ERR_INVALID, "args is NULL");
+  probe = *args; probe.workspace = nullptr; probe.workspace_bytes = 0;
+  if (int rc = baseline_fwd_args(&probe, &a, &bucket)) return rc;
+  size_t need = 0;
+  if (int rc = pat_fwd_workspace_bytes(&a, &need)) return rc;
+  *bytes = need + baseline_tables_bytes(args->batch);
+  return PAT_OK;
+}
+
+int pat_paged_decode_baseline_launch(const pat_baseline_args* args, void* hip_stream) {
+  pat_fwd_args a; pat_fwd_bucket bucket;
+  size_t need = 0;
+  if (int rc = pat_paged_decode_baseline_workspace_bytes(args, &need)) return rc;
+  if (args->workspace == nullptr || args->workspace_bytes < need)
+    return pat::fail(PAT_ERR_WORKSPACE, "workspace too small: need " + std::to_string(need) + " bytes, got " +
+                                            std::to_string(args->workspace_bytes));
+  if (reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
+    return pat::fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  if (int rc = baseline_fwd_args(args, &a, &bucket)) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const int n = args->batch;
+  hipLaunchKernelGGL(pat_baseline_tables_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                     const_cast<int32_t*>(bucket.q_table), const_cast<int32_t*>(bucket.num_seqs),
+                     const_cast<int32_t*>(bucket.rank), n);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return pat::hip_fail(e, "table fill kernel launch");
+  return pat_fwd_launch(&a, hip_stream);
+}
+
 }  // extern "C"

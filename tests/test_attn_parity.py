@@ -425,6 +425,25 @@ def test_reference_maximum_moves_with_sorted_keys():
     _assert_close("sorted keys", out, lse, ref_out, ref_lse, w.dtype)
 
 
+@pytest.mark.parametrize("name", ["c1", "c2", "c5b"])
+def test_paged_decode_baseline_matches_oracle(name):
+    # the prefix-oblivious comparator behind its own C-ABI entry point: block table + lengths in,
+    # one work item per request, same kernels
+    from pat_amd import paged_decode_baseline
+    print(f"[case] paged decode baseline {name}", flush=True)
+    dev = _device()
+    w = workloads.make(name, seed=9)
+    q, k, v = w.tensors(dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    lens = torch.tensor(w.seq_lens, dtype=torch.int32, device=dev)
+    paged_decode_baseline(q, k, v, w.padded_table().to(dev), lens, 1.0 / math.sqrt(w.head_dim), out,
+                          softmax_lse=lse, even_lengths=(name == "c5b"))
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"baseline {name}", out, lse, ref_out, ref_lse, w.dtype)
+
+
 def test_validation_errors_on_gpu_tensors():
     dev = _device()
     w = workloads.make("c1")

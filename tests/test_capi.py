@@ -130,3 +130,27 @@ def test_tree_handles_and_errors():
     nv = _lib.NodeView()
     assert lib.pat_tree_node(h, 5, C.byref(nv)) == _lib.PAT_ERR_INDEX
     lib.pat_tree_destroy(h)
+
+
+def test_baseline_workspace_and_errors_without_a_gpu():
+    lib = _lib.load()
+    fake = 0x10000
+    a = _lib.BaselineArgs()
+    a.dtype, a.batch, a.heads, a.kv_heads, a.head_dim = _lib.PAT_DTYPE_F16, 32, 64, 8, 128
+    a.page_size, a.num_pages, a.max_blocks = 16, 8192, 256
+    a.q = a.k = a.v = a.out = a.block_table = a.seq_lens = fake
+    a.q_stride = (C.c_int64 * 3)(8192, 8192, 128)
+    a.o_stride = (C.c_int64 * 3)(8192, 8192, 128)
+    a.k_stride = (C.c_int64 * 3)(16 * 8 * 128, 8 * 128, 128)
+    a.v_stride = (C.c_int64 * 3)(16 * 8 * 128, 8 * 128, 128)
+    a.block_table_stride, a.softmax_scale = 256, 0.088
+    need = C.c_size_t()
+    assert lib.pat_paged_decode_baseline_workspace_bytes(C.byref(a), C.byref(need)) == 0
+    # partial rows of 4096-token requests (>= 2 chunks) plus the three per-request tables
+    assert need.value >= 32 * 64 * 2 * (128 + 1) * 4 + 3 * 32 * 4
+    assert lib.pat_paged_decode_baseline_launch(C.byref(a), None) == _lib.PAT_ERR_WORKSPACE
+    a.max_blocks = 0
+    assert lib.pat_paged_decode_baseline_workspace_bytes(C.byref(a), C.byref(need)) == _lib.PAT_ERR_INVALID
+    assert "max_blocks" in _lib.last_error()
+    a.max_blocks, a.kv_heads = 256, 5
+    assert lib.pat_paged_decode_baseline_workspace_bytes(C.byref(a), C.byref(need)) == _lib.PAT_ERR_INVALID
