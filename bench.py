@@ -224,11 +224,13 @@ def main() -> None:
         "config": {"workload": f"{a.workload}: {WORKLOAD_TEXT[a.workload]}", "batch": w.batch,
                    "heads": w.heads, "kv_heads": w.kv_heads, "head_dim": w.head_dim, "page_size": w.page_size,
                    "seed": a.seed, "unique_kv_tokens": w.unique_tokens, "total_kv_tokens": w.total_tokens,
-                   "kv_cache_copies_rotated": copies},
+                   "kv_cache_copies_rotated": copies, "tree": w.tree},
         "us_per_call": round(ms_per_step * 1e3, 3),
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "unique_kv_bytes": unique_bytes,
         "oblivious_kv_bytes": w.kv_bytes(w.total_tokens),
+        # what the plan's work items read between them (L2 serves the re-reads of shared nodes)
+        "plan_kv_bytes": w.kv_bytes(int(sum(int(kv.sum()) for kv in info.kv_in_CTAs))),
         "event_us": {"call_median": round(median(call_ms) * 1e3, 3), "split_mean": round(split_mean_ms * 1e3, 3),
                      "split_interval_mean": round(mean(split_ms) * 1e3, 3),
                      "merge_mean": round((mean(merge_ms) - event_overhead_ms) * 1e3, 3),
