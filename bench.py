@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 INFINITY_CACHE_BYTES = 256 << 20
 # HBM bytes per split-kernel launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by
 # the same counter's reading for a 1 GiB copy kernel (profiles/pat_split_kernel_<workload>.md)
-MEASURED_TRAFFIC_BYTES = {"c2": 95_800_000}
+MEASURED_TRAFFIC_BYTES = {"c2": 95_800_000, "c5b": 541_800_000}
 
 WORKLOAD_TEXT = {
     "c1": "8 req, 256 shared + 32 private tokens, 8/8 heads, d64, fp16",
