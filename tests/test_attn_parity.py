@@ -83,6 +83,30 @@ def test_workload_table_overload(name, dtype):
     _assert_close(f"{name}/{dtype}", out, lse, ref_out, ref_lse, dtype)
 
 
+@pytest.mark.parametrize("name", ["c5b", "c3"])
+def test_table_overload_with_even_hint(name):
+    # bucket_flags is a hint: on c5b (equal lengths) it is true and selects a kv head per wave on
+    # long boxes, on c3 (ragged leaves) it is false; the result must not depend on it
+    print(f"[case] workload {name} table overload with PAT_BUCKET_EVEN on every bucket", flush=True)
+    from pat_amd._lib import PAT_BUCKET_EVEN
+    dev = _device()
+    w = workloads.make(name, seed=4)
+    q, k, v = w.tensors(dev)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+    ki.to_tensor(device=dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                             ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                             ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, None, softmax_lse=lse,
+                             slot_tables=ki.slot_tables, bucket_flags=[PAT_BUCKET_EVEN] * len(ki.MNWs))
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"{name}/even hint", out, lse, ref_out, ref_lse, w.dtype)
+
+
 @pytest.mark.parametrize("kind", ["naive", "compute_model", "sorted"])
 def test_other_plans_of_the_python_scheduler(kind):
     # plans the kernels see less often: the per-node plan of naive_schedule (no merging, many small
