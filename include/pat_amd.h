@@ -271,13 +271,16 @@ int pat_fwd_validate(const pat_fwd_args* args);
 
 /* Bytes of device scratch pat_fwd_launch needs for these arguments (partial
  * outputs + partial LSE; the reference allocates the equivalent per call at
- * csrc/api.h:217-229). Depends only on sizes, never on device data. */
+ * csrc/api.h:217-229). Depends only on sizes, pointers' alignment and strides, never on
+ * device data. 0 when every row has a single partial slot (max_split_per_seq 1 and no box
+ * longer than a chunk): the launch then writes `out` from its first kernel, as the reference
+ * does for max_split_per_seq 1 (csrc/api.h:230-238), and `workspace` may be NULL. */
 int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
 
 /* prefix_attn_with_kvcache(...)   csrc/bindings.cpp:7-72 -> csrc/api.h:110-295
- * Enqueues the split-KV kernels and the merge kernel on `hip_stream`
- * (a hipStream_t; NULL = the null stream) of the current device and returns
- * without synchronising. */
+ * Enqueues the split-KV kernel and (unless the workspace size is 0, see above) the merge
+ * kernel on `hip_stream` (a hipStream_t; NULL = the null stream) of the current device and
+ * returns without synchronising. */
 int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
 
 /* Description of the launch geometry chosen for `args` (for benchmarks/tests). */

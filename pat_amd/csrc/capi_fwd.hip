@@ -55,6 +55,7 @@ struct Geometry {
   int bucket_chunks[kMaxBuckets] = {0};
   int bucket_heads_per_wg[kMaxBuckets] = {0};   // 1, or kWaves: one kv head per wave
   int64_t total_wgs = 0;
+  bool direct = false;       // one slot per row: the split kernel writes `out`, no workspace, no merge kernel
 };
 
 int check_args(const pat_fwd_args* a) {
@@ -189,6 +190,26 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
       chunk = std::max(chunk, c);
     }
   }
+  // No sequence sits in two boxes (max_split_per_seq 1: a batch without shared prefixes, 27 boxes
+  // or more): with one chunk per box every row has a single partial slot and the split kernel
+  // writes `out` itself, which saves the second launch and the partial rows. Measured on 32..256
+  // independent requests of 64..2000 tokens: never slower than cutting the boxes, 10-30 % faster
+  // below 64 requests. Boxes longer than a chunk can be are cut as before, and so are launches
+  // of fewer boxes than CUs per kv head (explicit plans for small batches).
+  bool single_slot = false;
+  if (a->max_split_per_seq == 1 && !env_chunk && !env_tall) {
+    int64_t widest = 0;
+    for (int i = 0; i < a->num_buckets; ++i)
+      if (a->buckets[i].num_boxes > 0) widest = std::max<int64_t>(widest, (int64_t)a->buckets[i].max_blocks * page);
+    int64_t boxes = 0;
+    for (int i = 0; i < a->num_buckets; ++i) boxes += a->buckets[i].num_boxes;
+    // (with fewer boxes than one per CU and kv head, cutting them is what fills the device)
+    if (widest > 0 && round_unit(widest) <= std::min<int64_t>(cap, kMaxChunk) && boxes * a->kv_heads >= kNumCUs) {
+      chunk = std::max(chunk, widest);
+      tall = std::max(tall, widest);
+      single_slot = true;
+    }
+  }
   g->chunk = (int)std::min(round_unit(chunk), cap);
   g->tall_chunk = (int)std::min(round_unit(tall), cap);
   g->chunks_per_rank = 1;
@@ -258,6 +279,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
       const int64_t n = ceil_div64(tok, std::min(round_unit(want), cap));
       const int64_t c = std::min(round_unit(ceil_div64(tok, n)), cap);   // n even pieces of the widest box
       if (n > kMaxChunksPerRank) continue;
+      if (single_slot && n > 1) continue;   // (one chunk per box is worth as much, and keeps the launch single-slot)
       // an even bucket (caller's hint) has no stragglers: one such workgroup per CU is enough
       const int64_t need_i = (a->buckets[i].flags & PAT_BUCKET_EVEN) && !forced ? std::min<int64_t>(need, kNumCUs) : need;
       if ((int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need_i) continue;
@@ -276,6 +298,12 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     }
   }
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
+  // One slot per row (no sequence in two boxes, no box in two chunks): nothing to merge, the
+  // split kernel stores the rows in `out` itself (8-byte stores: needs `out` laid out for them).
+  // PAT_DIRECT_OUT=0 keeps the two-kernel route (tests).
+  g->direct = g->num_slots == 1 && reinterpret_cast<uintptr_t>(a->out) % 8 == 0 && a->o_stride[0] % 4 == 0 &&
+              a->o_stride[2] % 4 == 0;
+  if (const char* env = std::getenv("PAT_DIRECT_OUT")) g->direct = g->direct && std::atoi(env) != 0;
   if (g->total_wgs > (int64_t)kGridX * 65535 || g->total_wgs >= INT32_MAX)
     return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   // the kernels index partial rows with 32-bit integers
@@ -287,6 +315,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 size_t workspace_need(const pat_fwd_args* a, const Geometry& g) {
+  if (g.direct) return 0;
   const size_t rows = (size_t)a->batch * a->heads * g.num_slots;
   return align256(rows * a->head_dim * sizeof(float)) + align256(rows * sizeof(float));
 }
@@ -330,10 +359,10 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   Geometry g;
   if (int rc = plan_geometry(args, &g)) return rc;
   const size_t need = workspace_need(args, g);
-  if (args->workspace == nullptr || args->workspace_bytes < need)
+  if (need > 0 && (args->workspace == nullptr || args->workspace_bytes < need))
     return fail(PAT_ERR_WORKSPACE, "workspace too small: need " + std::to_string(need) + " bytes, got " +
                                        std::to_string(args->workspace_bytes));
-  if (reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
+  if (need > 0 && reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
     return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
 
@@ -346,6 +375,11 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   std::memset(&sp, 0, sizeof(sp));
   sp.q = args->q; sp.k = args->k; sp.v = args->v;
   sp.o_part = o_part; sp.lse_part = lse_part;
+  sp.direct = g.direct ? 1 : 0;
+  if (g.direct) {
+    sp.out = args->out; sp.lse_out = args->lse_out;
+    sp.o_stride_b = args->o_stride[0]; sp.o_stride_h = args->o_stride[2];
+  }
   sp.q_stride_b = args->q_stride[0]; sp.q_stride_h = args->q_stride[2];
   sp.k_stride_page = args->k_stride[0]; sp.k_stride_slot = args->k_stride[1]; sp.k_stride_h = args->k_stride[2];
   sp.v_stride_page = args->v_stride[0]; sp.v_stride_slot = args->v_stride[1]; sp.v_stride_h = args->v_stride[2];
@@ -398,6 +432,8 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
     const hipError_t e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), stream);
     if (e != hipSuccess) return hip_fail(e, "hipEventRecord(split_done_event)");
   }
+
+  if (g.direct) return PAT_OK;   // the rows are in `out` already
 
   MergeParams mp;
   std::memset(&mp, 0, sizeof(mp));

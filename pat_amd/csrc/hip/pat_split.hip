@@ -185,12 +185,44 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   // first partial slot of (my row, this box); -1: the row is not to be written
   const int my_slot0 = row_ok ? (my_seq_raw * p.heads + my_hq) * p.num_slots + my_ord * p.chunks_per_rank : -1;
 
+  // ---- where a finished row goes ---------------------------------------------------------
+  // Normally into its partial slot (fp32, merged by the second kernel). A launch in which every
+  // row has exactly one slot (no sequence in two boxes, no box in two chunks) has nothing to
+  // merge: its rows go straight to `out` in the output type (the reference does the same when
+  // max_split_per_seq is 1, csrc/api.h:230-238). A row's first slot index is then its
+  // (sequence, head) pair.
+  const bool direct = p.direct != 0;
+  auto row_out = [&](int slot0) -> T* {
+    const int s_ = slot0 / p.heads;
+    return (T*)p.out + (int64_t)s_ * p.o_stride_b + (int64_t)(slot0 - s_ * p.heads) * p.o_stride_h;
+  };
+  auto put4 = [&](float* part, T* out, f32x4 v) {
+    if (direct) {
+      typedef T tx4 __attribute__((ext_vector_type(4)));
+      *(tx4*)out = tx4{(T)v[0], (T)v[1], (T)v[2], (T)v[3]};
+    } else {
+      *(f32x4*)part = v;
+    }
+  };
+  auto put_lse = [&](int64_t prow, float lse) {
+    if (!direct) p.lse_part[prow] = lse;
+    else if (p.lse_out != nullptr) p.lse_out[prow] = lse;
+  };
+
   // ---- slots of this box that no workgroup will fill are marked empty (-inf) ------------
   {
     const bool empty = t_begin >= kv;
     const int first = empty ? chunk : chunk + 1;
     const int last = (chunk == bk.chunks - 1) ? p.chunks_per_rank : chunk + 1;  // exclusive
-    if ((shared_tiles || head_per_wave || wave == 0) && g == 0 && my_slot0 >= 0)
+    if (direct) {
+      // (one chunk per box: only a box without tokens gets here; its rows are zero, LSE -inf)
+      if (empty && (shared_tiles || head_per_wave || wave == 0) && my_slot0 >= 0) {
+        T* o = row_out(my_slot0) + g * 4;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) put4(nullptr, o + db * 16, f32x4{0.f, 0.f, 0.f, 0.f});
+        if (g == 0) put_lse(my_slot0, neg_inf());
+      }
+    } else if ((shared_tiles || head_per_wave || wave == 0) && g == 0 && my_slot0 >= 0)
       for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
 #ifdef PAT_TRACE
     if (empty && p.trace && tid == 0) {
@@ -406,9 +438,10 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       const int64_t prow = (int64_t)my_slot0 + chunk;
       const float inv = 1.f / l_run;
       float* dst = p.o_part + prow * D + g * 4;
+      T* o = direct ? row_out(my_slot0) + g * 4 : nullptr;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
-      if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+      for (int db = 0; db < DB; ++db) put4(dst + db * 16, o + db * 16, acc_o[db] * inv);
+      if (g == 0) put_lse(prow, (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f);
     }
   } else {
     // ====================== short box: KV steps split over the 4 waves ========================
@@ -490,9 +523,10 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         const int64_t prow = (int64_t)my_slot0 + chunk;
         const float inv = 1.f / l_run;
         float* dst = p.o_part + prow * D + g * 4;
+        T* o = direct ? row_out(my_slot0) + g * 4 : nullptr;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) *(f32x4*)(dst + db * 16) = acc_o[db] * inv;
-        if (g == 0) p.lse_part[prow] = (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f;
+        for (int db = 0; db < DB; ++db) put4(dst + db * 16, o + db * 16, acc_o[db] * inv);
+        if (g == 0) put_lse(prow, (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f);
       }
     } else {
     // combine the 4 waves' states through LDS and write the partial
@@ -521,16 +555,17 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       const float inv = 1.f / wsum;
       const int64_t prow = (int64_t)cslot0 + chunk;
       float* dst = p.o_part + prow * D + ccol;
+      T* od = direct ? row_out(cslot0) + ccol : nullptr;
 #pragma unroll
       for (int c = 0; c < D / 16; c += 4) {
         f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < kWaves; ++w)
           o += *(const f32x4*)(cbuf + (w * 16 + crow) * OROW + ccol + c) * wgt[w];
-        *(f32x4*)(dst + c) = o * inv;
+        put4(dst + c, od + c, o * inv);
       }
       if ((tid & 15) == 0)
-        p.lse_part[prow] = (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f;
+        put_lse(prow, (mmax + __builtin_amdgcn_logf(wsum)) * 0.6931471805599453f);
     }
     }   // combine
   }

@@ -107,6 +107,53 @@ def test_table_overload_with_even_hint(name):
     _assert_close(f"{name}/even hint", out, lse, ref_out, ref_lse, w.dtype)
 
 
+@pytest.mark.parametrize("case", ["combine", "head_per_wave", "tall_identical"])
+def test_single_slot_launch_writes_out_directly(case, monkeypatch):
+    # every row has one partial slot (no sequence in two boxes, no box in two chunks): the split
+    # kernel stores `out` itself, needs no workspace and no merge kernel follows
+    # (csrc/api.h:230-238 does the same for max_split_per_seq == 1). All three epilogues. (Batches
+    # of 27 boxes or more: below that the balancer halves boxes and every row has two slots.)
+    print(f"[case] direct output, {case}", flush=True)
+    from pat_amd import _prefix_attn
+    dev = _device()
+    if case == "combine":          # few boxes of a few steps: 4 waves share a box, states combined in LDS
+        w = workloads.independent("direct-a", 32, 300, 32, 8, 128, torch.bfloat16, 5)
+    elif case == "head_per_wave":  # many one-step boxes: a kv head per wave
+        w = workloads.independent("direct-b", 256, 100, 16, 8, 64, torch.float16, 6)
+    else:                          # 32 groups of 8 requests with the same pages: boxes of 32 rows
+        base = workloads.independent("direct-c", 32, 200, 32, 8, 128, torch.float16, 7)
+        w = workloads.Workload("direct-c", 32, 8, 128, torch.float16, base.page_size, [200] * 256,
+                               [list(base.rows[i // 8]) for i in range(256)], base.num_blocks, 32 * 200, 7)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    assert info.max_split_per_seq == 1
+    lt = info.launch_tables()
+
+    def run(direct):
+        monkeypatch.setenv("PAT_DIRECT_OUT", "1" if direct else "0")
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+        L = _prefix_attn._prepare(q, k, v, info.num_split_per_seq, lt["q_tables"], lt["block_tables"],
+                                  lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
+                                  info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                                  1.0 / math.sqrt(w.head_dim), out, lse, lt.get("slot_tables"), lt.get("flags"))
+        assert (L.need == 0) == direct, f"direct {direct}: workspace {L.need} bytes"
+        _prefix_attn._run(L, dev)
+        torch.cuda.synchronize()
+        return out, lse
+
+    out_d, lse_d = run(True)
+    out_m, lse_m = run(False)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"direct/{case}", out_d, lse_d, ref_out, ref_lse, w.dtype)
+    assert torch.equal(out_d, out_m), "direct store and merge kernel must agree bit for bit"
+    assert torch.equal(lse_d, lse_m)
+
+
 @pytest.mark.parametrize("kind", ["naive", "compute_model", "sorted"])
 def test_other_plans_of_the_python_scheduler(kind):
     # plans the kernels see less often: the per-node plan of naive_schedule (no merging, many small
