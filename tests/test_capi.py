@@ -119,6 +119,44 @@ def test_geometry_and_workspace_are_consistent():
     assert lib.pat_fwd_launch(C.byref(a), None) == _lib.PAT_ERR_WORKSPACE
 
 
+def test_single_slot_launch_needs_no_workspace(monkeypatch):
+    # no sequence in two boxes (max_split_per_seq 1), every box one chunk, a box per CU and kv head:
+    # the launch writes `out` from its first kernel (csrc/api.h:230-238) and needs no scratch
+    lib = _lib.load()
+    fake = 0x10000
+
+    def plan(boxes, blocks, **over):
+        b = (_lib.FwdBucket * 1)()
+        b[0].q_table = b[0].block_table = b[0].num_seqs = b[0].rank = b[0].kv = fake
+        b[0].q_table_stride, b[0].block_table_stride = 1, blocks
+        b[0].num_boxes, b[0].max_seqs, b[0].max_blocks = boxes, 1, blocks
+        b[0].mnw[0], b[0].mnw[1], b[0].mnw[2] = 16, 128, 1
+        kw = dict(batch=boxes, max_split_per_seq=1, max_seqs_in_box=1, max_blocks_in_box=blocks, num_buckets=1,
+                  buckets=C.cast(b, C.POINTER(_lib.FwdBucket)))
+        kw.update(over)
+        a = _args(**kw)
+        a._keep = b
+        g, need = _lib.FwdGeometry(), C.c_size_t()
+        assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
+        assert lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)) == 0
+        return g, need.value
+
+    monkeypatch.delenv("PAT_DIRECT_OUT", raising=False)
+    g, need = plan(64, 100)                       # 64 boxes of 1600 tokens, 8 kv heads: 512 workgroups
+    assert (g.chunks_per_rank, g.num_slots, need) == (1, 1, 0)
+    g, need = plan(64, 100, out=fake + 2)         # `out` not 8-byte aligned: the two-kernel route
+    assert g.num_slots == 1 and need > 0
+    g, need = plan(64, 100, max_split_per_seq=2)  # some sequence sits in two boxes
+    assert need > 0
+    g, need = plan(16, 100)                       # 128 workgroups: cutting the boxes fills the device
+    assert g.chunks_per_rank > 1 and need > 0
+    g, need = plan(64, 200)                       # 3200 tokens: longer than a chunk can be
+    assert g.chunks_per_rank > 1 and need > 0
+    monkeypatch.setenv("PAT_DIRECT_OUT", "0")
+    g, need = plan(64, 100)
+    assert g.num_slots == 1 and need > 0
+
+
 def test_tree_handles_and_errors():
     lib = _lib.load()
     h = C.c_void_p()
