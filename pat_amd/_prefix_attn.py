@@ -381,8 +381,12 @@ def _raw_stream(index: int) -> int:
 
 def _run(L: _Launch, device: torch.device) -> None:
     # scratch for the partial results, from torch's caching allocator on the current stream
-    ws = torch.empty(L.need, dtype=torch.uint8, device=device)
-    L.args.workspace = ws.data_ptr()
+    # (none for a single-slot launch, which writes `out` from its first kernel)
+    if L.need:
+        ws = torch.empty(L.need, dtype=torch.uint8, device=device)
+        L.args.workspace = ws.data_ptr()
+    else:
+        L.args.workspace = None
     L.args.workspace_bytes = L.need
     rc = _lib.load().pat_fwd_launch(C.byref(L.args), C.c_void_p(_raw_stream(device.index)))
     if rc:
