@@ -154,6 +154,32 @@ def test_single_slot_launch_writes_out_directly(case, monkeypatch):
     assert torch.equal(lse_d, lse_m)
 
 
+@pytest.mark.parametrize("pad", [8, 2])
+def test_single_slot_launch_with_strided_out(pad):
+    # `out` as a view with padded head rows: 8 extra elements keep 8-byte stores possible (direct
+    # route), 2 do not (the launch falls back to partial slots + merge); same result either way
+    print(f"[case] direct output into a strided view, head rows padded by {pad}", flush=True)
+    from pat_amd import _prefix_attn
+    dev = _device()
+    w = workloads.independent("direct-s", 48, 400, 32, 8, 128, torch.float16, 9)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    big = torch.full((w.batch, 1, w.heads, w.head_dim + pad), float("nan"), dtype=q.dtype, device=dev)
+    out = big[..., :w.head_dim]
+    lse = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    info = tree.kernel_info
+    L = next(iter(info._launch_cache.values()))
+    assert (L.need == 0) == (pad == 8)
+    assert torch.isnan(big[..., w.head_dim:]).all(), "the padding of the view must stay untouched"
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"direct/strided{pad}", out, lse, ref_out, ref_lse, w.dtype)
+
+
 @pytest.mark.parametrize("kind", ["naive", "compute_model", "sorted"])
 def test_other_plans_of_the_python_scheduler(kind):
     # plans the kernels see less often: the per-node plan of naive_schedule (no merging, many small
