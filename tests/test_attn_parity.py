@@ -559,3 +559,40 @@ def test_validation_errors_on_gpu_tensors():
     with pytest.raises(RuntimeError, match="64 / 128"):
         prefix_attn_with_kvcache(q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous(), tree,
                                  0.125, out[..., :32].contiguous())
+
+
+def test_randomized_workloads_fixed_seed():
+    # 120 workloads drawn from a fixed seed: independent requests, one shared prefix, three-level trees
+    # and irregular forests over 8 head configurations, both head dims and element types; small ones
+    # (the oracle runs on the CPU). Batches without sharing of 27 requests or more take the
+    # single-slot route, the rest every other route the launch geometry knows.
+    import numpy as np
+    dev = _device()
+    rng = np.random.default_rng(20240607)
+    head_cfgs = [(8, 8), (16, 8), (32, 8), (64, 8), (16, 16), (32, 32), (8, 4), (16, 4)]
+    done = 0
+    while done < 120:
+        h, hk = head_cfgs[rng.integers(len(head_cfgs))]
+        d = int(rng.choice([64, 128]))
+        dtype = [torch.float16, torch.bfloat16][rng.integers(2)]
+        kind, seed = int(rng.integers(4)), int(rng.integers(1 << 30))
+        if kind == 0:
+            w = workloads.independent("rnd", int(rng.integers(1, 200)), int(rng.integers(1, 2600)), h, hk, d, dtype, seed)
+        elif kind == 1:
+            w = workloads.shared_prefix("rnd", int(rng.integers(2, 150)), int(rng.integers(1, 200)) * 16, 1,
+                                        int(rng.integers(2, 700)), h, hk, d, dtype, seed)
+        elif kind == 2:
+            mids = int(rng.integers(1, 5))
+            w = workloads.three_level("rnd", mids * int(rng.integers(2, 30)), int(rng.integers(1, 100)) * 16, mids,
+                                      int(rng.integers(1, 40)) * 16, 1, int(rng.integers(2, 400)), h, hk, d, dtype, seed)
+        else:
+            w = workloads.forest("rnd", int(rng.integers(4, 100)), int(rng.integers(1, 5)), h, hk, d, dtype, seed,
+                                 root_range=(64, 1500), inner_range=(16, 300), leaf_range=(1, 200))
+        if w.kv_bytes(w.total_tokens) > 1.5e8:
+            continue
+        print(f"[case] random {done}: kind {kind} batch {w.batch} heads {h}/{hk} d {d} {dtype} seed {seed}", flush=True)
+        q, k, v = w.tensors(dev)
+        out, lse = _run_tree(w, q, k, v)
+        ref_out, ref_lse = _oracle(w, q, k, v)
+        _assert_close(f"random {done}", out, lse, ref_out, ref_lse, dtype)
+        done += 1
