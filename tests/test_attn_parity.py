@@ -522,14 +522,16 @@ def test_reference_maximum_moves_with_sorted_keys():
     _assert_close("sorted keys", out, lse, ref_out, ref_lse, w.dtype)
 
 
-@pytest.mark.parametrize("name", ["c1", "c2", "c5b"])
+@pytest.mark.parametrize("name", ["c1", "c2", "c5b", "independent"])
 def test_paged_decode_baseline_matches_oracle(name):
     # the prefix-oblivious comparator behind its own C-ABI entry point: block table + lengths in,
-    # one work item per request, same kernels
+    # one work item per request, same kernels ("independent": 64 requests of 500 tokens, which the
+    # launch serves with one slot per row and no merge kernel)
     from pat_amd import paged_decode_baseline
     print(f"[case] paged decode baseline {name}", flush=True)
     dev = _device()
-    w = workloads.make(name, seed=9)
+    w = (workloads.independent("ind", 64, 500, 32, 8, 128, torch.bfloat16, 9) if name == "independent"
+         else workloads.make(name, seed=9))
     q, k, v = w.tensors(dev)
     out = torch.full_like(q, float("nan"))
     lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
