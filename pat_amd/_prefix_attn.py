@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes as C
-from typing import List, Optional, Sequence, Union
+from typing import List, Optional, Union
 
 import numpy as np
 import torch
