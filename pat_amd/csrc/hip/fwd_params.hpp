@@ -37,9 +37,6 @@ struct SplitParams {
   const void* v;
   float* o_part;     // [batch, heads, num_slots, head_dim] fp32, normalised partial outputs
   float* lse_part;   // [batch, heads, num_slots] fp32, natural-log LSE of each partial (-inf = empty)
-  void* out;         // direct launches: [batch, 1, heads, head_dim] in the element type, else unused
-  float* lse_out;    // direct launches: optional [batch, heads] fp32
-  int64_t o_stride_b, o_stride_h;              // elements
   int64_t q_stride_b, q_stride_h;              // elements
   int64_t k_stride_page, k_stride_slot, k_stride_h;
   int64_t v_stride_page, v_stride_slot, v_stride_h;
@@ -48,7 +45,6 @@ struct SplitParams {
   int32_t chunks_per_rank;  // slots reserved per CTA_rank
   int32_t num_slots;        // max_split_per_seq * chunks_per_rank
   int32_t max_split;
-  int32_t direct;           // 1: num_slots is 1 and rows are written to `out` (no merge kernel follows)
   int32_t total_items;      // workgroups over all buckets: (box, chunk) items x head groups, head group fastest
   float scale_log2;         // softmax_scale * log2(e)
   int32_t num_buckets;
@@ -58,6 +54,12 @@ struct SplitParams {
   long long* trace;         // debug builds only: 8 timestamps/ids per workgroup
 #endif
   BucketDev bucket[kMaxBuckets];
+  // single-slot launches (every row has one partial slot; no merge kernel follows): the rows go
+  // to `out`. Kept behind the fields every launch reads, whose offsets the bucket search relies on.
+  void* out;         // [batch, 1, heads, head_dim] in the element type
+  float* lse_out;    // optional [batch, heads] fp32
+  int64_t o_stride_b, o_stride_h;              // elements
+  int32_t direct;    // 1: such a launch
 };
 
 struct MergeParams {

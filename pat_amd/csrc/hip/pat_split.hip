@@ -72,7 +72,8 @@ __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 #ifndef PAT_OCC
 #define PAT_OCC 3     // resident workgroups per CU the register budget is sized for
 #endif
-template <typename T, int D>
+// DIRECT instances serve launches in which every row has one partial slot: they store `out`.
+template <typename T, int D, bool DIRECT>
 __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -191,7 +192,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   // merge: its rows go straight to `out` in the output type (the reference does the same when
   // max_split_per_seq is 1, csrc/api.h:230-238). A row's first slot index is then its
   // (sequence, head) pair.
-  const bool direct = p.direct != 0;
+  constexpr bool direct = DIRECT;
   auto row_out = [&](int slot0) -> T* {
     const int s_ = slot0 / p.heads;
     return (T*)p.out + (int64_t)s_ * p.o_stride_b + (int64_t)(slot0 - s_ * p.heads) * p.o_stride_h;
@@ -585,10 +586,14 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
 }
 
 // Host launcher: picks the instance for (element type, head_dim).
+template <bool DIRECT>
+static void (*split_instance(bool bf16, int head_dim))(const SplitParams) {
+  if (bf16) return head_dim == 64 ? pat_split_kernel<__bf16, 64, DIRECT> : pat_split_kernel<__bf16, 128, DIRECT>;
+  return head_dim == 64 ? pat_split_kernel<_Float16, 64, DIRECT> : pat_split_kernel<_Float16, 128, DIRECT>;
+}
+
 hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const SplitParams& params) {
-  void (*fn)(const SplitParams);
-  if (bf16) fn = head_dim == 64 ? pat_split_kernel<__bf16, 64> : pat_split_kernel<__bf16, 128>;
-  else fn = head_dim == 64 ? pat_split_kernel<_Float16, 64> : pat_split_kernel<_Float16, 128>;
+  void (*fn)(const SplitParams) = params.direct ? split_instance<true>(bf16, head_dim) : split_instance<false>(bf16, head_dim);
   const unsigned wgs = (unsigned)params.total_items;
   const dim3 grid(wgs < (unsigned)kGridX ? wgs : (unsigned)kGridX, (wgs + kGridX - 1) / kGridX);
   hipLaunchKernelGGL(fn, grid, dim3(kThreads), 0, stream, params);
