@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PAT_ABI_VERSION 1
+#define PAT_ABI_VERSION 2
 
 /* ---- status codes ------------------------------------------------------- */
 #define PAT_OK 0
@@ -113,6 +113,13 @@ typedef struct pat_plan_view {
   int32_t max_split_per_seq;
   int32_t max_seqs_in_box;          /* KernelInfo.max_seqs_in_CTA             */
   int32_t max_blocks_in_box;        /* KernelInfo.max_blocks_in_CTA           */
+  /* Not part of the reference plan: the number of boxes of THIS plan that contain each
+   * sequence (= 1 + the sequence's largest q_slot) and its maximum. num_split_per_seq is the
+   * reference's counter, which keeps counting over repeated pack calls on one tree
+   * (prefix_attn/prefix_tree.py:149 resets it only when the tree is rebuilt); a launch that
+   * files partial results by q_slot merges num_boxes_per_seq of them. */
+  const int32_t* num_boxes_per_seq; /* [batch]                                */
+  int32_t max_boxes_per_seq;
 } pat_plan_view;
 
 /* PrefixTree(block_size)                     prefix_attn/prefix_tree.py:48-59 */
@@ -184,6 +191,9 @@ typedef struct pat_flat_plan {
   int32_t max_split_per_seq, max_seqs_in_box, max_blocks_in_box;
   int64_t total;               /* int32 elements the buffer needs                        */
   int64_t num_split_per_seq;   /* offset, [batch]                                        */
+  int64_t num_boxes_per_seq;   /* offset, [batch]: see pat_plan_view.num_boxes_per_seq   */
+  int32_t max_boxes_per_seq;
+  int32_t pad_;
   int64_t launch_order[PAT_MAX_FLAT_BUCKETS];
   pat_flat_bucket buckets[PAT_MAX_FLAT_BUCKETS];
   pat_flat_bucket launch[PAT_MAX_FLAT_BUCKETS];
@@ -282,6 +292,44 @@ int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
  * kernel on `hip_stream` (a hipStream_t; NULL = the null stream) of the current device and
  * returns without synchronising. */
 int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
+
+/* Partial-result slots for a plan that carries none (pat_fwd_bucket.q_slot == NULL), e.g. the
+ * tensors of KernelInfo.to_tensor passed positionally as benchmark/benchmark_kernel.py:247-265
+ * does. Filing partial results by CTA_rank, as the reference kernel does
+ * (csrc/block_info.h:29-35), loses one wherever the reference scheduler hands the same rank to two
+ * boxes of a sequence (irregular forests). pat_fwd_derive_slots runs one small kernel on
+ * `hip_stream` that reads the q_tables / num_seqs of args->buckets and writes into `buffer`
+ * (device memory, 256-byte aligned, pat_fwd_slots_bytes() bytes):
+ *   int32 [batch]                      boxes of the plan that contain each sequence, at offset 0
+ *   int32 [num_boxes, q_table_stride]  per bucket i, at element offset bucket_offsets[i] (host
+ *                                      array [num_buckets], filled by the call): for every
+ *                                      (box, sequence) the box's ordinal among that sequence's
+ *                                      boxes, buckets in order, boxes in order
+ * The caller then launches with buckets[i].q_slot = buffer + bucket_offsets[i] and
+ * num_split_per_seq = buffer. The result depends on the plan's contents: derive again after the
+ * q_tables change. */
+int pat_fwd_slots_bytes(const pat_fwd_args* args, size_t* bytes);
+int pat_fwd_derive_slots(const pat_fwd_args* args, void* buffer, size_t buffer_bytes,
+                         int64_t* bucket_offsets, void* hip_stream);
+
+/* Overrides of the launch geometry: a tuning and test aid, process-wide, not meant to change
+ * while launches are in flight on other threads. 0 / -1 = automatic, as noted per field. The
+ * initial values come from the environment variables PAT_CHUNK_TOKENS, PAT_TALL_CHUNK_TOKENS,
+ * PAT_HEAD_PER_WAVE_TOKENS, PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS,
+ * PAT_EQUALIZE_CHUNKS, PAT_DIRECT_OUT, read once; pat_fwd_set_tuning(NULL) reads them again. */
+typedef struct pat_fwd_tuning {
+  int32_t chunk_tokens;              /* KV tokens per workgroup, boxes <= 16 rows (0: automatic)   */
+  int32_t tall_chunk_tokens;         /* same for boxes of 17..64 rows (0: automatic)                */
+  int32_t head_per_wave_tokens;      /* widest box of a bucket that runs a kv head per wave         */
+                                     /* (-1: automatic, 0: never)                                   */
+  int32_t head_per_wave_long_tokens; /* chunk of long boxes run a kv head per wave (0: automatic)   */
+  int64_t head_per_wave_long_wgs;    /* such workgroups a bucket needs for that (-1: automatic)     */
+  int32_t equalize_chunks;           /* even chunks per box: -1 automatic, 0 never, 1 always        */
+  int32_t direct_out;                /* single-slot launches write `out` from the split kernel:     */
+                                     /* -1 / 1 when possible, 0 never                               */
+} pat_fwd_tuning;
+int pat_fwd_set_tuning(const pat_fwd_tuning* tuning);
+int pat_fwd_get_tuning(pat_fwd_tuning* out);
 
 /* Description of the launch geometry chosen for `args` (for benchmarks/tests). */
 typedef struct pat_fwd_geometry {

@@ -12,6 +12,8 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpat_amd.so")
 
+ABI_VERSION = 2
+
 PAT_OK = 0
 PAT_ERR_INVALID = -1
 PAT_ERR_VALUE = -2
@@ -49,7 +51,8 @@ class PlanView(C.Structure):
     _fields_ = [("num_buckets", C.c_int32), ("batch", C.c_int32),
                 ("buckets", C.POINTER(BucketView)), ("num_split_per_seq", i32p),
                 ("max_split_per_seq", C.c_int32), ("max_seqs_in_box", C.c_int32),
-                ("max_blocks_in_box", C.c_int32)]
+                ("max_blocks_in_box", C.c_int32), ("num_boxes_per_seq", i32p),
+                ("max_boxes_per_seq", C.c_int32)]
 
 
 class FlatBucket(C.Structure):
@@ -66,6 +69,7 @@ class FlatPlan(C.Structure):
     _fields_ = [("num_buckets", C.c_int32), ("num_launch_buckets", C.c_int32), ("batch", C.c_int32),
                 ("max_split_per_seq", C.c_int32), ("max_seqs_in_box", C.c_int32),
                 ("max_blocks_in_box", C.c_int32), ("total", C.c_int64), ("num_split_per_seq", C.c_int64),
+                ("num_boxes_per_seq", C.c_int64), ("max_boxes_per_seq", C.c_int32), ("pad_", C.c_int32),
                 ("launch_order", C.c_int64 * MAX_FLAT_BUCKETS), ("buckets", FlatBucket * MAX_FLAT_BUCKETS),
                 ("launch", FlatBucket * MAX_FLAT_BUCKETS)]
 
@@ -108,6 +112,17 @@ class FwdArgs(C.Structure):
                 ("split_done_event", C.c_void_p)]
 
 
+class FwdTuning(C.Structure):
+    _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
+                ("head_per_wave_tokens", C.c_int32), ("head_per_wave_long_tokens", C.c_int32),
+                ("head_per_wave_long_wgs", C.c_int64), ("equalize_chunks", C.c_int32),
+                ("direct_out", C.c_int32)]
+
+    @classmethod
+    def automatic(cls) -> "FwdTuning":
+        return cls(0, 0, -1, 0, -1, -1, -1)
+
+
 class FwdGeometry(C.Structure):
     _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
                 ("chunks_per_rank", C.c_int32), ("num_slots", C.c_int32),
@@ -132,6 +147,10 @@ SYMBOLS = {
     "pat_fwd_validate": (C.c_int, [C.POINTER(FwdArgs)]),
     "pat_fwd_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_launch": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "pat_fwd_slots_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
+    "pat_fwd_derive_slots": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_size_t, i64p, C.c_void_p]),
+    "pat_fwd_set_tuning": (C.c_int, [C.POINTER(FwdTuning)]),
+    "pat_fwd_get_tuning": (C.c_int, [C.POINTER(FwdTuning)]),
     "pat_paged_decode_baseline_workspace_bytes": (C.c_int, [C.POINTER(BaselineArgs), C.POINTER(C.c_size_t)]),
     "pat_paged_decode_baseline_launch": (C.c_int, [C.POINTER(BaselineArgs), C.c_void_p]),
     "pat_fwd_geometry_of": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(FwdGeometry)]),
@@ -155,8 +174,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.pat_abi_version() != 1:
-        raise ImportError(f"{LIB_PATH}: ABI version {lib.pat_abi_version()} != 1, rebuild it")
+    if lib.pat_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.pat_abi_version()} != {ABI_VERSION}, rebuild it")
     _lib = lib
     return lib
 

@@ -48,6 +48,10 @@ class KernelInfo:
         self.MNWs: List[List[int]] = []
         self.num_split_per_seq: torch.Tensor = torch.empty(0, dtype=torch.int32)
         self.max_split_per_seq = 0
+        # not in the reference: boxes of this plan per sequence (what a launch by slot_tables merges;
+        # num_split_per_seq keeps counting over repeated pack_schedule calls, as the reference's does)
+        self.num_boxes_per_seq: torch.Tensor = torch.empty(0, dtype=torch.int32)
+        self.max_boxes_per_seq = 0
         self.max_seqs_in_CTA = 0
         self.max_blocks_in_CTA = 0
         self._launch_cache: dict = {}
@@ -147,6 +151,7 @@ class KernelInfo:
         self.kv_in_CTAs = [move(t) for t in self.kv_in_CTAs]
         self.slot_tables = [move(t) for t in self.slot_tables]
         self.num_split_per_seq = move(self.num_split_per_seq)
+        self.num_boxes_per_seq = move(self.num_boxes_per_seq)
         if self._launch_tables is not None:
             self._launch_tables = {name: (ts if name in ("MNWs", "flags") else [move(t) for t in ts])
                                    for name, ts in self._launch_tables.items()}
@@ -167,6 +172,7 @@ class KernelInfo:
         ki._flat_layout = layout
         ki._flat = host
         ki.max_split_per_seq = layout.max_split_per_seq
+        ki.max_boxes_per_seq = layout.max_boxes_per_seq
         ki.max_seqs_in_CTA = layout.max_seqs_in_box
         ki.max_blocks_in_CTA = layout.max_blocks_in_box
         ki._bind(host)
@@ -187,6 +193,7 @@ class KernelInfo:
                     "kv_in_CTAs": flat[f.kv:f.kv + n]}
 
         self.num_split_per_seq = flat[lay.num_split_per_seq:lay.num_split_per_seq + lay.batch]
+        self.num_boxes_per_seq = flat[lay.num_boxes_per_seq:lay.num_boxes_per_seq + lay.batch]
         for name in self._PER_BOX:
             setattr(self, name, [])
         self.MNWs, self._launch_order, self._launch_parts = [], [], []
@@ -233,7 +240,10 @@ class KernelInfo:
             ki._block_lens.append(np.ctypeslib.as_array(bk.block_len, shape=(n,)).copy() if n else np.zeros(0, np.int32))
         ki.num_split_per_seq = torch.from_numpy(
             np.ctypeslib.as_array(view.num_split_per_seq, shape=(view.batch,)).copy())
+        ki.num_boxes_per_seq = torch.from_numpy(
+            np.ctypeslib.as_array(view.num_boxes_per_seq, shape=(view.batch,)).copy())
         ki.max_split_per_seq = view.max_split_per_seq
+        ki.max_boxes_per_seq = view.max_boxes_per_seq
         ki.max_seqs_in_CTA = view.max_seqs_in_box
         ki.max_blocks_in_CTA = view.max_blocks_in_box
         ki._sort_for_launch()
@@ -362,13 +372,27 @@ def _prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, M
         _check(lse.is_cuda and lse.dtype == torch.float32 and lse.is_contiguous() and lse.numel() == b * h,
                "softmax_lse must be a contiguous CUDA float32 tensor with batch_size * n_heads elements")
         a.lse_out = lse.data_ptr()
+    derived = None
+    if slot_tables is None and int(max_split) > 1:
+        # A plan without slot tables (the reference's call form): CTA_rank is not unique per sequence
+        # on irregular forests, so the ordinals are derived from the q_tables on the device, once per
+        # prepared launch (the cache keys hold the tables' version counters).
+        sbytes = C.c_size_t(0)
+        _lib.check(lib.pat_fwd_slots_bytes(C.byref(a), C.byref(sbytes)))
+        derived = torch.empty(sbytes.value, dtype=torch.uint8, device=q.device)
+        offsets = (C.c_int64 * max(nb, 1))()
+        _lib.check(lib.pat_fwd_derive_slots(C.byref(a), C.c_void_p(derived.data_ptr()), sbytes.value, offsets,
+                                            C.c_void_p(_raw_stream(q.device.index))))
+        for i in range(nb):
+            L.buckets[i].q_slot = derived.data_ptr() + 4 * offsets[i]
+        a.num_split_per_seq = derived.data_ptr()
     need = C.c_size_t(0)
     _lib.check(lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)))
     L.args, L.need = a, need.value
     # plan tensors stay referenced as long as the prepared launch does; q/k/v/out are the
     # caller's for the duration of the call only
     L.keep = (num_split, list(q_tables), list(block_tables), list(num_seqs), list(ranks), list(kvs),
-              None if slot_tables is None else list(slot_tables))
+              None if slot_tables is None else list(slot_tables), derived)
     L.workspace = None
     return L
 
@@ -403,7 +427,7 @@ def _table_key(q, k, v, out, lse, vals, slots, flags=None):
         def ident(t):
             return (t.data_ptr(), tuple(t.shape), t.stride())
         def small(t):   # plan tensors: 1-D, or 2-D with contiguous rows (checked when the launch is built)
-            return (t.data_ptr(), t.numel(), t.stride(0))
+            return (t.data_ptr(), t.numel(), t.stride(0), t._version)
         lists = tuple(tuple(small(t) for t in vals[name]) for name in
                       ("query_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs"))
         return (ident(q), ident(k), ident(v), ident(out), q.dtype, None if lse is None else ident(lse),
@@ -468,9 +492,11 @@ def prefix_attn_with_kvcache(q: torch.Tensor, k_cache_paged: torch.Tensor, v_cac
             L = info._launch_cache.get(key)
             if L is None:
                 lt = info.launch_tables()
-                L = _prepare(q, k_cache_paged, v_cache_paged, info.num_split_per_seq, lt["q_tables"],
+                # partial results are filed by slot_tables: the launch merges each sequence's boxes of
+                # THIS plan (num_split_per_seq counts on over repeated pack_schedule calls)
+                L = _prepare(q, k_cache_paged, v_cache_paged, info.num_boxes_per_seq, lt["q_tables"],
                              lt["block_tables"], lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"],
-                             lt["MNWs"], info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                             lt["MNWs"], info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
                              vals["softmax_scale"], out, lse, lt.get("slot_tables"), lt.get("flags"))
                 if len(info._launch_cache) >= 256:
                     info._launch_cache.clear()

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 #include "capi_error.hpp"
@@ -39,10 +40,35 @@ inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = 
 // (16,128,1) for pages under 32 tokens, csrc/api.h:177-181).
 inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 2 : 4); }
 
-// Widest box (tokens) of a bucket whose workgroups serve one kv head per wave
-// (PAT_HEAD_PER_WAVE_TOKENS overrides; 0 switches the mode off).
-int64_t head_per_wave_tokens(bool oversubscribed) {
-  if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_TOKENS")) return std::atoll(env);
+// Overrides of the launch geometry (pat_fwd_set_tuning). The defaults come from the environment
+// variables PAT_CHUNK_TOKENS, PAT_TALL_CHUNK_TOKENS, PAT_HEAD_PER_WAVE_TOKENS,
+// PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS, PAT_EQUALIZE_CHUNKS and
+// PAT_DIRECT_OUT, read once per process: no launch reads the environment.
+pat_fwd_tuning env_tuning() {
+  pat_fwd_tuning t;
+  t.chunk_tokens = 0; t.tall_chunk_tokens = 0; t.head_per_wave_tokens = -1;
+  t.head_per_wave_long_wgs = -1; t.head_per_wave_long_tokens = 0; t.equalize_chunks = -1; t.direct_out = -1;
+  if (const char* e = std::getenv("PAT_CHUNK_TOKENS")) t.chunk_tokens = std::atoi(e);
+  if (const char* e = std::getenv("PAT_TALL_CHUNK_TOKENS")) t.tall_chunk_tokens = std::atoi(e);
+  if (const char* e = std::getenv("PAT_HEAD_PER_WAVE_TOKENS")) t.head_per_wave_tokens = std::atoi(e);
+  if (const char* e = std::getenv("PAT_HEAD_PER_WAVE_LONG_WGS")) t.head_per_wave_long_wgs = std::atoll(e);
+  if (const char* e = std::getenv("PAT_HEAD_PER_WAVE_LONG_TOKENS")) t.head_per_wave_long_tokens = std::atoi(e);
+  if (const char* e = std::getenv("PAT_EQUALIZE_CHUNKS")) t.equalize_chunks = std::atoi(e) != 0;
+  if (const char* e = std::getenv("PAT_DIRECT_OUT")) t.direct_out = std::atoi(e) != 0;
+  return t;
+}
+std::mutex g_tuning_mutex;
+pat_fwd_tuning g_tuning;
+bool g_tuning_set = false;
+pat_fwd_tuning tuning() {
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  if (!g_tuning_set) { g_tuning = env_tuning(); g_tuning_set = true; }
+  return g_tuning;
+}
+
+// Widest box (tokens) of a bucket whose workgroups serve one kv head per wave (0: mode off).
+int64_t head_per_wave_tokens(const pat_fwd_tuning& t, bool oversubscribed) {
+  if (t.head_per_wave_tokens >= 0) return t.head_per_wave_tokens;
   return oversubscribed ? 256 : 128;
 }
 
@@ -122,6 +148,9 @@ int check_args(const pat_fwd_args* a) {
       return fail(PAT_ERR_INVALID, "plan table row stride too large" + at);
     if ((int64_t)b.max_seqs * ratio > 64)
       return fail(PAT_ERR_INVALID, "a box may pack at most 64 rows (sequences x heads per kv head)" + at);
+    // the tile label is the bucket's row class: a box with more rows than its label would lose them
+    if ((int64_t)b.max_seqs * ratio > 16 * row_tiles(b.mnw[0]))
+      return fail(PAT_ERR_INVALID, "a box packs more rows (sequences x heads per kv head) than its bucket's tile_q" + at);
   }
   return PAT_OK;
 }
@@ -135,8 +164,9 @@ int check_args(const pat_fwd_args* a) {
 //  * boxes of 17..64 rows walk the chunk step by step with all 4 waves (one row tile each) and
 //    write 16..32 KB of partial output per workgroup: their chunk is at least 256 tokens, and
 //    longer when they alone would still fill the device.
-// PAT_CHUNK_TOKENS / PAT_TALL_CHUNK_TOKENS override the two sizes (tuning aid).
+// pat_fwd_tuning.chunk_tokens / tall_chunk_tokens override the two sizes (tuning aid).
 int plan_geometry(const pat_fwd_args* a, Geometry* g) {
+  const pat_fwd_tuning tune = tuning();
   const int page = a->page_size;
   const int64_t unit = (int64_t)page * kStepTokens / gcd64(page, kStepTokens);  // lcm(page, 32)
   auto round_unit = [&](int64_t c) { return std::max<int64_t>(unit, ceil_div64(c, unit) * unit); };
@@ -147,9 +177,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     const int64_t w = (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
     if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w; else tall_work += w;
   }
-  int64_t chunk = 0, tall = 0;
-  if (const char* env = std::getenv("PAT_CHUNK_TOKENS")) chunk = std::atoll(env);
-  if (const char* env = std::getenv("PAT_TALL_CHUNK_TOKENS")) tall = std::atoll(env);
+  int64_t chunk = tune.chunk_tokens, tall = tune.tall_chunk_tokens;
   const bool env_tall = tall > 0, env_chunk = chunk > 0;
   if (chunk <= 0) {
     // whole multiples of 128 tokens: the 4 waves of a workgroup get the same number of steps,
@@ -221,8 +249,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     const int64_t wgs = (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, is_tall ? g->tall_chunk : g->chunk)) * a->kv_heads;
     (is_tall ? kind_tall_wgs : kind_short_wgs) += wgs;
   }
-  int equalize = -1;   // PAT_EQUALIZE_CHUNKS=0/1 overrides the rule below (tuning aid)
-  if (const char* env = std::getenv("PAT_EQUALIZE_CHUNKS")) equalize = std::atoi(env) != 0;
+  const int equalize = tune.equalize_chunks;   // 0/1 override the rule below (tuning aid)
   for (int i = 0; i < a->num_buckets; ++i) {
     const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
     int64_t c = row_tiles(a->buckets[i].mnw[0]) > 1 ? g->tall_chunk : g->chunk;
@@ -250,7 +277,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   if (g->total_wgs >= 2 * kNumCUs && a->kv_heads % kWaves == 0) {
     // up to 256 tokens when the launch does not fit on the device at once, up to 128 when it
     // does (every workgroup is resident from the start and the longest chain sets the time)
-    const int64_t limit = head_per_wave_tokens(g->total_wgs > (int64_t)kResidentWgsPerCU * kNumCUs);
+    const int64_t limit = head_per_wave_tokens(tune, g->total_wgs > (int64_t)kResidentWgsPerCU * kNumCUs);
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
       if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= limit) {
@@ -264,18 +291,18 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   // 4 adjacent heads of the same tokens (1 KB contiguous per token instead of 256 bytes), which
   // streams ~9 % faster; each wave walks its chunk alone, one step in flight, so this needs enough
   // queued workgroups to keep every CU's waves busy to the end (a launch that fits at once ends
-  // on its longest chains instead: c3 +11 %, c2 +37 %). PAT_HEAD_PER_WAVE_LONG_WGS overrides the
-  // number of such workgroups a bucket must have (0: always, tuning and tests).
+  // on its longest chains instead: c3 +11 %, c2 +37 %). pat_fwd_tuning.head_per_wave_long_wgs overrides
+  // the number of such workgroups a bucket must have (0: always, tuning and tests).
   if (a->kv_heads % kWaves == 0) {
     int64_t need = 2 * (int64_t)kResidentWgsPerCU * kNumCUs;
     bool forced = false;
-    if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_WGS")) { need = std::atoll(env); forced = true; }
+    if (tune.head_per_wave_long_wgs >= 0) { need = tune.head_per_wave_long_wgs; forced = true; }
     bool changed = false;
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
       if (row_tiles(a->buckets[i].mnw[0]) != 1 || g->bucket_heads_per_wg[i] != 1 || tok <= 256) continue;
       int64_t want = kLongHeadPerWaveChunk;
-      if (const char* env = std::getenv("PAT_HEAD_PER_WAVE_LONG_TOKENS")) want = std::max<int64_t>(32, std::atoll(env));
+      if (tune.head_per_wave_long_tokens > 0) want = std::max<int64_t>(32, tune.head_per_wave_long_tokens);
       const int64_t n = ceil_div64(tok, std::min(round_unit(want), cap));
       const int64_t c = std::min(round_unit(ceil_div64(tok, n)), cap);   // n even pieces of the widest box
       if (n > kMaxChunksPerRank) continue;
@@ -300,10 +327,9 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   g->num_slots = g->chunks_per_rank * a->max_split_per_seq;
   // One slot per row (no sequence in two boxes, no box in two chunks): nothing to merge, the
   // split kernel stores the rows in `out` itself (8-byte stores: needs `out` laid out for them).
-  // PAT_DIRECT_OUT=0 keeps the two-kernel route (tests).
+  // pat_fwd_tuning.direct_out = 0 keeps the two-kernel route (tests).
   g->direct = g->num_slots == 1 && reinterpret_cast<uintptr_t>(a->out) % 8 == 0 && a->o_stride[0] % 4 == 0 &&
-              a->o_stride[2] % 4 == 0;
-  if (const char* env = std::getenv("PAT_DIRECT_OUT")) g->direct = g->direct && std::atoi(env) != 0;
+              a->o_stride[2] % 4 == 0 && tune.direct_out != 0;
   if (g->total_wgs > (int64_t)kGridX * 65535 || g->total_wgs >= INT32_MAX)
     return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
   // the kernels index partial rows with 32-bit integers
@@ -353,22 +379,19 @@ int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes) {
   return PAT_OK;
 }
 
-int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
-  using namespace pat;
-  if (int rc = check_args(args)) return rc;
-  Geometry g;
-  if (int rc = plan_geometry(args, &g)) return rc;
-  const size_t need = workspace_need(args, g);
-  if (need > 0 && (args->workspace == nullptr || args->workspace_bytes < need))
-    return fail(PAT_ERR_WORKSPACE, "workspace too small: need " + std::to_string(need) + " bytes, got " +
-                                       std::to_string(args->workspace_bytes));
-  if (need > 0 && reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
-    return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+}  // extern "C"
+
+// ---- the two launches of one call --------------------------------------------------------------
+namespace pat {
+namespace {
+
+// Everything pat_fwd_launch does after the argument checks: `workspace` holds the partial results.
+int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, void* hip_stream) {
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
 
   const size_t rows = (size_t)args->batch * args->heads * g.num_slots;
-  float* o_part = static_cast<float*>(args->workspace);
-  float* lse_part = reinterpret_cast<float*>(static_cast<char*>(args->workspace) +
+  float* o_part = static_cast<float*>(workspace);
+  float* lse_part = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                              align256(rows * args->head_dim * sizeof(float)));
 
   SplitParams sp;
@@ -418,10 +441,6 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
     }
     sp.num_buckets = nb;
     sp.total_items = (int32_t)items;
-#ifdef PAT_TRACE
-    sp.trace = nullptr;
-    if (const char* env = std::getenv("PAT_TRACE_PTR")) sp.trace = reinterpret_cast<long long*>(std::strtoull(env, nullptr, 0));
-#endif
     if (items > 0) {
       const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, sp);
       if (e != hipSuccess) return hip_fail(e, "split kernel launch");
@@ -444,6 +463,128 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   mp.chunks_per_rank = g.chunks_per_rank; mp.num_slots = g.num_slots; mp.max_split = args->max_split_per_seq;
   const hipError_t e = launch_merge(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, mp);
   if (e != hipSuccess) return hip_fail(e, "merge kernel launch");
+  return PAT_OK;
+}
+
+// ---- partial-result slots for plans that carry none ---------------------------------------------
+// Ordinal of every (box, sequence) among the boxes of that sequence, in launch order (buckets in
+// order, boxes in order), and the number of boxes per sequence: what the planner emits as q_slot /
+// num_boxes_per_seq, derived on the device from the q_tables of a plan that came without them.
+struct SlotBucket {
+  const int32_t* q_table;
+  const int32_t* num_seqs;
+  int32_t* q_slot;
+  int32_t q_stride, num_boxes, max_seqs;
+};
+struct SlotParams {
+  SlotBucket bucket[kMaxBuckets];
+  int32_t* num_boxes_per_seq;
+  int32_t num_buckets, batch;
+};
+
+// One wave per sequence walks every q_table entry of the plan, 64 at a time.
+__global__ void __launch_bounds__(256) pat_slot_kernel(const SlotParams p) {
+  const int lane = threadIdx.x & 63;
+  const int s = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (s >= p.batch) return;
+  int count = 0;
+  for (int b = 0; b < p.num_buckets; ++b) {
+    const SlotBucket bk = p.bucket[b];
+    const int entries = bk.num_boxes * bk.max_seqs;
+    for (int base = 0; base < entries; base += 64) {
+      const int e = base + lane;
+      bool live = false, hit = false;
+      int at = 0;
+      if (e < entries) {
+        const int box = e / bk.max_seqs, j = e - box * bk.max_seqs;
+        at = box * bk.q_stride + j;
+        const int q = bk.q_table[at];
+        live = j < bk.num_seqs[box] && (unsigned)q < (unsigned)p.batch;
+        hit = live && q == s;
+      }
+      const unsigned long long mask = __ballot(hit);
+      if (hit) bk.q_slot[at] = count + __popcll(mask & ((1ull << lane) - 1ull));
+      if (e < entries && !live && s == 0) bk.q_slot[at] = 0;   // padding: defined, never used
+      count += __popcll(mask);
+    }
+  }
+  if (lane == 0) p.num_boxes_per_seq[s] = count;
+}
+
+}  // namespace
+}  // namespace pat
+
+extern "C" {
+
+int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
+  using namespace pat;
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  const size_t need = workspace_need(args, g);
+  if (need > 0 && (args->workspace == nullptr || args->workspace_bytes < need))
+    return fail(PAT_ERR_WORKSPACE, "workspace too small: need " + std::to_string(need) + " bytes, got " +
+                                       std::to_string(args->workspace_bytes));
+  if (need > 0 && reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
+    return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  return launch_core(args, g, args->workspace, hip_stream);
+}
+
+int pat_fwd_slots_bytes(const pat_fwd_args* args, size_t* bytes) {
+  if (bytes == nullptr) return pat::fail(PAT_ERR_INVALID, "bytes is NULL");
+  if (int rc = pat::check_args(args)) return rc;
+  size_t n = pat::align256((size_t)args->batch * sizeof(int32_t));
+  for (int i = 0; i < args->num_buckets; ++i)
+    n += pat::align256((size_t)args->buckets[i].num_boxes * (size_t)args->buckets[i].q_table_stride * sizeof(int32_t));
+  *bytes = n;
+  return PAT_OK;
+}
+
+int pat_fwd_derive_slots(const pat_fwd_args* args, void* buffer, size_t buffer_bytes, int64_t* bucket_offsets,
+                         void* hip_stream) {
+  using namespace pat;
+  size_t need = 0;
+  if (int rc = pat_fwd_slots_bytes(args, &need)) return rc;
+  if (buffer == nullptr || bucket_offsets == nullptr) return fail(PAT_ERR_INVALID, "buffer / bucket_offsets is NULL");
+  if (buffer_bytes < need)
+    return fail(PAT_ERR_WORKSPACE, "slot buffer too small: need " + std::to_string(need) + " bytes, got " +
+                                       std::to_string(buffer_bytes));
+  if (reinterpret_cast<uintptr_t>(buffer) % 256 != 0) return fail(PAT_ERR_WORKSPACE, "slot buffer must be 256-byte aligned");
+  SlotParams sp;
+  std::memset(&sp, 0, sizeof(sp));
+  sp.num_boxes_per_seq = static_cast<int32_t*>(buffer);
+  sp.batch = args->batch;
+  size_t at = align256((size_t)args->batch * sizeof(int32_t));
+  int nb = 0;
+  for (int i = 0; i < args->num_buckets; ++i) {
+    const pat_fwd_bucket& b = args->buckets[i];
+    bucket_offsets[i] = (int64_t)(at / sizeof(int32_t));
+    if (b.num_boxes > 0 && b.max_seqs > 0) {
+      if ((int64_t)b.num_boxes * b.max_seqs >= INT32_MAX) return fail(PAT_ERR_INVALID, "q_table too large");
+      SlotBucket& d = sp.bucket[nb++];
+      d.q_table = b.q_table; d.num_seqs = b.num_seqs;
+      d.q_slot = reinterpret_cast<int32_t*>(static_cast<char*>(buffer) + at);
+      d.q_stride = (int32_t)b.q_table_stride; d.num_boxes = b.num_boxes; d.max_seqs = b.max_seqs;
+    }
+    at += align256((size_t)b.num_boxes * (size_t)b.q_table_stride * sizeof(int32_t));
+  }
+  sp.num_buckets = nb;
+  hipLaunchKernelGGL(pat_slot_kernel, dim3((unsigned)((args->batch + 3) / 4)), dim3(256), 0,
+                     static_cast<hipStream_t>(hip_stream), sp);
+  if (const hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "slot kernel launch");
+  return PAT_OK;
+}
+
+int pat_fwd_set_tuning(const pat_fwd_tuning* t) {
+  std::lock_guard<std::mutex> lock(pat::g_tuning_mutex);
+  pat::g_tuning = t ? *t : pat::env_tuning();
+  pat::g_tuning_set = true;
+  return PAT_OK;
+}
+
+int pat_fwd_get_tuning(pat_fwd_tuning* out) {
+  if (out == nullptr) return pat::fail(PAT_ERR_INVALID, "out is NULL");
+  *out = pat::tuning();
   return PAT_OK;
 }
 

@@ -126,6 +126,8 @@ int pat_tree_plan(const pat_tree* tree, pat_plan_view* out) {
   out->max_split_per_seq = p.max_split;
   out->max_seqs_in_box = p.max_seqs_in_box;
   out->max_blocks_in_box = p.max_blocks_in_box;
+  out->num_boxes_per_seq = p.num_boxes_per_seq.data();
+  out->max_boxes_per_seq = p.max_boxes;
   return PAT_OK;
 }
 
@@ -141,6 +143,7 @@ static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* 
   layout->num_buckets = nb;
   layout->batch = (int32_t)p.num_split_per_seq.size();
   layout->max_split_per_seq = p.max_split;
+  layout->max_boxes_per_seq = p.max_boxes;
   layout->max_seqs_in_box = p.max_seqs_in_box;
   layout->max_blocks_in_box = p.max_blocks_in_box;
 
@@ -178,6 +181,7 @@ static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* 
   int64_t at = 0;
   auto take = [&](int64_t n) { const int64_t o = at; at += n; return o; };
   layout->num_split_per_seq = take(layout->batch);
+  layout->num_boxes_per_seq = take(layout->batch);
   auto place = [&](pat_flat_bucket& f, const pat::Bucket& bk, int rows, int width, int parent, int first) {
     std::memcpy(f.mnw, bk.mnw, sizeof(f.mnw));
     f.num_boxes = rows; f.max_seqs = bk.max_seqs; f.max_blocks = width; f.parent = parent; f.first = first;
@@ -215,6 +219,7 @@ static int flat_plan_impl(const pat_tree* tree, pat_flat_plan* layout, int32_t* 
 
   // contents
   std::copy(p.num_split_per_seq.begin(), p.num_split_per_seq.end(), dst + layout->num_split_per_seq);
+  std::copy(p.num_boxes_per_seq.begin(), p.num_boxes_per_seq.end(), dst + layout->num_boxes_per_seq);
   auto rows_to = [&](int32_t* out, const std::vector<int32_t>& table, int src_width, int width,
                      const int32_t* ord, int lo, int hi) {
     for (int i = lo; i < hi; ++i) {

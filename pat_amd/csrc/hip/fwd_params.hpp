@@ -50,9 +50,6 @@ struct SplitParams {
   int32_t num_buckets;
   uint32_t hpp_magic;       // ceil(2^32 / (page_size / 16)): h / (page_size / 16) == umulhi(h, hpp_magic) for h < 2^16; unused when page_size / 16 is a power of two
   int32_t item_begin[kMaxBuckets];  // copy of bucket[i].item_begin at fixed offsets (INT32_MAX past the end)
-#ifdef PAT_TRACE
-  long long* trace;         // debug builds only: 8 timestamps/ids per workgroup
-#endif
   BucketDev bucket[kMaxBuckets];
   // single-slot launches (every row has one partial slot; no merge kernel follows): the rows go
   // to `out`. Kept behind the fields every launch reads, whose offsets the bucket search relies on.

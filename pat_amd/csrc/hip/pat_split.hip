@@ -99,12 +99,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   __shared__ float s_m[kWaves][16];
   __shared__ float s_l[kWaves][16];
 
-#ifdef PAT_TRACE
-  long long tr[6] = {wall_clock64(), 0, 0, 0, 0, 0};
-#define PAT_STAMP(i) tr[i] = wall_clock64()
-#else
-#define PAT_STAMP(i)
-#endif
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -137,9 +131,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const int chunk = local / bk.num_boxes;
   const int box = local - chunk * bk.num_boxes;
   if (chunk >= bk.chunks) return;
-#ifdef PAT_TRACE
-  const int wg = wg_id;
-#endif
 
   // Boxes of up to 16 rows: the 4 waves split the chunk's steps, each on wave-private tiles.
   // Taller boxes: wave w owns rows 16w..16w+15, all waves walk the same steps on tiles shared
@@ -178,7 +169,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
   if (R == 0) return;
   const bool has_rows = row0 < R;   // false: a wave that only helps loading shared tiles
-  PAT_STAMP(1);
 
   const bool row_ok = (row0 + n < R) && ((unsigned)my_seq_raw < (unsigned)p.batch) &&
                       ((unsigned)my_ord < (unsigned)p.max_split);
@@ -225,14 +215,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
       }
     } else if ((shared_tiles || head_per_wave || wave == 0) && g == 0 && my_slot0 >= 0)
       for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
-#ifdef PAT_TRACE
-    if (empty && p.trace && tid == 0) {
-      long long* t = p.trace + (long long)wg * 8;
-      const long long now = wall_clock64();
-      t[0] = tr[0]; t[1] = now; t[2] = now; t[3] = now; t[4] = now; t[5] = 0; t[6] = 0;
-      t[7] = ((long long)bi << 48) | ((long long)box << 24) | chunk;
-    }
-#endif
     if (empty) return;
   }
   const int t_end = (kv < t_begin + bk.chunk_tokens) ? kv : t_begin + bk.chunk_tokens;
@@ -409,10 +391,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     for (int s = 0; s < PF; ++s)
       if (s < nsteps) fetch(s, kst[s], vst[s]);
     load_q();
-#ifdef PAT_TRACE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    PAT_STAMP(2);
-#endif
     for (int st0 = 0; st0 < nsteps; st0 += PF) {
 #pragma unroll
       for (int s = 0; s < PF; ++s) {
@@ -433,7 +411,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
                  stage + kStepTokens * RSK, t_begin + st * kStepTokens, []() {});
       }
     }
-    PAT_STAMP(3);
     l_run = sum_xor32(sum_xor16(l_run));
     if (my_slot0 >= 0) {
       const int64_t prow = (int64_t)my_slot0 + chunk;
@@ -493,10 +470,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         fetch_v(step0 + d * stride, vring[d]);
         fetch_k(step0 + d * stride, kring[d]);
       }
-#ifdef PAT_TRACE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    PAT_STAMP(2);
-#endif
     for (int st0 = step0; st0 < nsteps; st0 += DEPTH * stride) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
@@ -515,7 +488,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
                t_begin + st * kStepTokens, [&]() { if (more) fetch_k(nxt, kring[d]); });
       }
     }
-    PAT_STAMP(3);
     l_run = sum_xor32(sum_xor16(l_run));
 
     if (head_per_wave) {
@@ -570,19 +542,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     }
     }   // combine
   }
-#ifdef PAT_TRACE
-  if (p.trace && tid == 0) {
-    PAT_STAMP(4);
-    unsigned hw, xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    long long* t = p.trace + (long long)wg * 8;
-    for (int i = 0; i < 5; ++i) t[i] = tr[i];
-    t[5] = ((long long)xcc << 32) | hw;
-    t[6] = nsteps;
-    t[7] = ((long long)bi << 48) | ((long long)box << 24) | chunk;
-  }
-#endif
 }
 
 // Host launcher: picks the instance for (element type, head_dim).

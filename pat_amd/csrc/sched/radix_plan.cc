@@ -358,6 +358,8 @@ void RadixPlanner::bucketize(const std::vector<Box>& boxes,
   if (plan.num_split_per_seq.empty())
     throw SchedError{PAT_ERR_VALUE, "max() arg is an empty sequence"};
   plan.max_split = *std::max_element(plan.num_split_per_seq.begin(), plan.num_split_per_seq.end());
+  plan.max_boxes = *std::max_element(boxes_seen.begin(), boxes_seen.end());
+  plan.num_boxes_per_seq = std::move(boxes_seen);
   for (const Box& b : boxes) {
     plan.max_seqs_in_box = std::max(plan.max_seqs_in_box, (int)b.seqs.size());
     plan.max_blocks_in_box = std::max(plan.max_blocks_in_box, (int)b.blocks.size());

@@ -71,6 +71,8 @@ struct Plan {
   std::vector<Bucket> buckets;
   std::vector<pat_bucket_view> views;
   std::vector<int32_t> num_split_per_seq;
+  std::vector<int32_t> num_boxes_per_seq;   // boxes of this plan that hold each sequence
+  int max_boxes = 0;
   int max_split = 0, max_seqs_in_box = 0, max_blocks_in_box = 0;
   bool valid = false;
 };

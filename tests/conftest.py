@@ -55,3 +55,23 @@ def golden_small():
 @pytest.fixture(scope="session")
 def golden_large():
     return load_golden("plans_large.json.gz")
+
+
+@pytest.fixture
+def tuning():
+    """Sets launch-geometry overrides of libpat_amd (pat_fwd_set_tuning) for one test:
+    `tuning(direct_out=0)`; the automatic values come back when the test ends."""
+    import ctypes as C
+    from pat_amd import _lib
+    lib = _lib.load()
+
+    def apply(**fields):
+        t = _lib.FwdTuning.automatic()
+        for name, value in fields.items():
+            assert hasattr(t, name), name
+            setattr(t, name, value)
+        assert lib.pat_fwd_set_tuning(C.byref(t)) == 0
+
+    yield apply
+    auto = _lib.FwdTuning.automatic()
+    lib.pat_fwd_set_tuning(C.byref(auto))

@@ -30,7 +30,10 @@ def _oracle(w, q, k, v):
 def _assert_close(name, out, lse, ref_out, ref_lse, dtype):
     err = (out.float().cpu() - ref_out.float()).abs().max().item()
     lerr = ((lse.cpu() - ref_lse).abs() / ref_lse.abs().clamp_min(1.0)).max().item()
-    print(f"[parity] {name}: max|out - ref| = {err:.3e} (tol {TOL[dtype]:.1e}), LSE rel = {lerr:.3e}", flush=True)
+    # the strictly relative figure as well: it is larger than the gated one only where |LSE| < 1
+    strict = ((lse.cpu() - ref_lse).abs() / ref_lse.abs().clamp_min(1e-30)).max().item()
+    print(f"[parity] {name}: max|out - ref| = {err:.3e} (tol {TOL[dtype]:.1e}), LSE rel = {lerr:.3e} "
+          f"(strictly relative {strict:.3e})", flush=True)
     assert err <= TOL[dtype], f"{name}: output error {err}"
     assert lerr <= LSE_RTOL, f"{name}: LSE error {lerr}"
 
@@ -83,6 +86,137 @@ def test_workload_table_overload(name, dtype):
     _assert_close(f"{name}/{dtype}", out, lse, ref_out, ref_lse, dtype)
 
 
+def _ragged_forest_workload(seed, heads, d, dtype):
+    import random
+    r = random.Random(seed)
+    nxt = [0]
+
+    def blocks(n):
+        out = list(range(nxt[0], nxt[0] + n)); nxt[0] += n
+        return out
+
+    rows, lens = [], []
+    for _ in range(5):                      # roots of very different lengths: the long-box cut fires
+        root = blocks(r.choice([3, 30, 150, 260]))
+        for _ in range(r.randint(1, 4)):
+            mid = root + blocks(r.randint(1, 12))
+            for _ in range(r.randint(1, 6)):
+                row = mid + blocks(r.randint(1, 9))
+                rows.append(row)
+                lens.append(len(row) * 16 - r.randint(0, 15))
+    perm = list(range(nxt[0])); r.shuffle(perm)
+    rows = [[perm[x] for x in row] for row in rows]
+    return workloads.Workload("ragged forest", heads[0], heads[1], d, dtype, 16, lens, rows, nxt[0], 0, seed)
+
+
+@pytest.mark.parametrize("case", ["c4", "ragged"])
+def test_reference_call_form_unchanged(case):
+    # exactly benchmark/benchmark_kernel.py:247-265: Python PrefixTree, KernelInfo.to_tensor, sixteen
+    # positional arguments, nothing else. On c4 at seed 0 the reference scheduler hands one CTA_rank
+    # to two boxes of a sequence 11 times (and 5 ranks are >= that sequence's num_split): filing
+    # partial results by rank would lose them, the binding derives collision-free slots itself.
+    print(f"[case] reference call form, {case}", flush=True)
+    dev = _device()
+    w = workloads.make("c4", seed=0) if case == "c4" else _ragged_forest_workload(5, (16, 4), 128, torch.float16)
+    q, k, v = w.tensors(dev)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+    if case == "c4":
+        # the hazard is really there: some sequence sees one rank twice
+        seen, twice = set(), 0
+        for qt, rk in zip(ki.q_tables, ki.CTA_ranks):
+            for row, rank in zip(qt, rk):
+                for s in row:
+                    twice += (s, rank) in seen
+                    seen.add((s, rank))
+        assert twice > 0
+    ki.to_tensor(device=dev)
+    out = torch.full_like(q, float("nan"))
+    prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                             ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                             ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, None)
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    out2 = torch.full_like(q, float("nan"))
+    prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                             ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                             ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out2, None, softmax_lse=lse)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    assert torch.equal(out, out2)
+    _assert_close(f"{case} reference call form", out, lse, ref_out, ref_lse, w.dtype)
+
+
+def test_second_pack_schedule_on_one_tree():
+    # the reference's per-sequence split counters count on over repeated pack_schedule calls; the
+    # launch merges the boxes of the current plan, whatever the counters say
+    print("[case] c3, pack_schedule twice on one tree", flush=True)
+    dev = _device()
+    w = workloads.make("c3", seed=1)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    first = tree.kernel_info.max_split_per_seq
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    assert tree.kernel_info.max_split_per_seq == 2 * first
+    tree.kernel_info.to_gpu(dev)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("c3 second pack", out, lse, ref_out, ref_lse, w.dtype)
+
+
+def test_merge_of_more_than_256_slots(tuning):
+    # five nested nodes -> every request sits in five boxes (naive_schedule: one box per node); with
+    # 32-token chunks the 2048-token root reserves 64 slots per box: 320 slots per row, so the
+    # merge kernel's loops past its 256 register-held slots run
+    print("[case] merge of 320 slots per row", flush=True)
+    import ctypes as C
+    from pat_amd import _lib, _prefix_attn
+    dev = _device()
+    nxt = [0]
+
+    def blocks(n):
+        out = list(range(nxt[0], nxt[0] + n)); nxt[0] += n
+        return out
+
+    root = blocks(128)
+    rows, lens = [], []
+    for i in range(16):
+        if i % 8 == 0:
+            a = blocks(4)
+        if i % 4 == 0:
+            b = blocks(4)
+        if i % 2 == 0:
+            c = blocks(2)
+        row = root + a + b + c + blocks(2)
+        rows.append(row)
+        lens.append(len(row) * 16 - 15)
+    w = workloads.Workload("nested", 8, 8, 64, torch.float16, 16, lens, rows, nxt[0], 0, 9)
+    q, k, v = w.tensors(dev)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    ki = t.naive_schedule(1)
+    assert ki.max_split_per_seq == 5
+    ki.to_tensor(device=dev)
+    tuning(chunk_tokens=32, tall_chunk_tokens=32)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    L = _prefix_attn._prepare(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                              ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                              ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, lse)
+    geo = _lib.FwdGeometry()
+    assert _lib.load().pat_fwd_geometry_of(C.byref(L.args), C.byref(geo)) == 0
+    assert geo.num_slots == 5 * 64
+    _prefix_attn._run(L, dev)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("320 slots", out, lse, ref_out, ref_lse, w.dtype)
+
+
 @pytest.mark.parametrize("name", ["c5b", "c3"])
 def test_table_overload_with_even_hint(name):
     # bucket_flags is a hint: on c5b (equal lengths) it is true and selects a kv head per wave on
@@ -108,7 +242,7 @@ def test_table_overload_with_even_hint(name):
 
 
 @pytest.mark.parametrize("case", ["combine", "head_per_wave", "tall_identical"])
-def test_single_slot_launch_writes_out_directly(case, monkeypatch):
+def test_single_slot_launch_writes_out_directly(case, tuning):
     # every row has one partial slot (no sequence in two boxes, no box in two chunks): the split
     # kernel stores `out` itself, needs no workspace and no merge kernel follows
     # (csrc/api.h:230-238 does the same for max_split_per_seq == 1). All three epilogues. (Batches
@@ -134,7 +268,7 @@ def test_single_slot_launch_writes_out_directly(case, monkeypatch):
     lt = info.launch_tables()
 
     def run(direct):
-        monkeypatch.setenv("PAT_DIRECT_OUT", "1" if direct else "0")
+        tuning(direct_out=1 if direct else 0)
         out = torch.full_like(q, float("nan"))
         lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
         L = _prefix_attn._prepare(q, k, v, info.num_split_per_seq, lt["q_tables"], lt["block_tables"],
@@ -394,7 +528,7 @@ def test_device_selftest_reports_no_mismatch():
 
 
 @pytest.mark.parametrize("heads,dtype", [((32, 8), torch.bfloat16), ((16, 16), torch.float16)])
-def test_large_ragged_batch_all_launch_modes(heads, dtype):
+def test_large_ragged_batch_all_launch_modes(heads, dtype, tuning):
     # a launch several times what fits on the device at once: short private tails (one kv head per
     # wave), mid-size shared nodes, a few long shared roots read by many 64-row boxes, boxes sorted
     # longest first for the launch
@@ -429,13 +563,8 @@ def test_large_ragged_batch_all_launch_modes(heads, dtype):
     _assert_close("large ragged", out, lse, ref_out, ref_lse, dtype)
     # the same batch with a kv head per wave on every bucket of <= 16-row boxes, long ones included
     # (the geometry a launch with thousands of such workgroups gets by itself)
-    import os
-    os.environ["PAT_HEAD_PER_WAVE_LONG_WGS"] = "0"
-    os.environ["PAT_HEAD_PER_WAVE_TOKENS"] = "256"
-    try:
-        out, lse = _run_tree(w, q, k, v)
-    finally:
-        del os.environ["PAT_HEAD_PER_WAVE_LONG_WGS"], os.environ["PAT_HEAD_PER_WAVE_TOKENS"]
+    tuning(head_per_wave_long_wgs=0, head_per_wave_tokens=256)
+    out, lse = _run_tree(w, q, k, v)
     _assert_close("large ragged, a kv head per wave", out, lse, ref_out, ref_lse, dtype)
 
 

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"libpat_amd.so does not export {name}"
     assert sorted(_lib.SYMBOLS) == names       # the ctypes table covers the header, no more, no less
-    assert lib.pat_abi_version() == 1
+    assert lib.pat_abi_version() == 2
 
 
 def _args(**over):
@@ -98,6 +98,12 @@ def test_validate_rejects_bad_bucket_and_strides():
     a.buckets[1].max_seqs = 32      # 32 sequences x 4 heads per kv head > 64 rows
     a.buckets[1].q_table_stride = 32
     assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "64 rows" in _lib.last_error()
+    a = _args()
+    a.buckets[1].max_seqs = 8       # 8 sequences x 4 heads = 32 rows in a bucket labelled tile_q 16
+    a.buckets[1].q_table_stride = 8
+    assert lib.pat_fwd_validate(C.byref(a)) == _lib.PAT_ERR_INVALID and "than its bucket's tile_q" in _lib.last_error()
+    a.buckets[1].mnw[0] = 32        # ... which a tile_q 32 bucket holds
+    assert lib.pat_fwd_validate(C.byref(a)) == 0
 
 
 def test_geometry_and_workspace_are_consistent():
@@ -119,7 +125,7 @@ def test_geometry_and_workspace_are_consistent():
     assert lib.pat_fwd_launch(C.byref(a), None) == _lib.PAT_ERR_WORKSPACE
 
 
-def test_single_slot_launch_needs_no_workspace(monkeypatch):
+def test_single_slot_launch_needs_no_workspace(tuning):
     # no sequence in two boxes (max_split_per_seq 1), every box one chunk, a box per CU and kv head:
     # the launch writes `out` from its first kernel (csrc/api.h:230-238) and needs no scratch
     lib = _lib.load()
@@ -141,7 +147,7 @@ def test_single_slot_launch_needs_no_workspace(monkeypatch):
         assert lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)) == 0
         return g, need.value
 
-    monkeypatch.delenv("PAT_DIRECT_OUT", raising=False)
+    tuning()
     g, need = plan(64, 100)                       # 64 boxes of 1600 tokens, 8 kv heads: 512 workgroups
     assert (g.chunks_per_rank, g.num_slots, need) == (1, 1, 0)
     g, need = plan(64, 100, out=fake + 2)         # `out` not 8-byte aligned: the two-kernel route
@@ -152,9 +158,30 @@ def test_single_slot_launch_needs_no_workspace(monkeypatch):
     assert g.chunks_per_rank > 1 and need > 0
     g, need = plan(64, 200)                       # 3200 tokens: longer than a chunk can be
     assert g.chunks_per_rank > 1 and need > 0
-    monkeypatch.setenv("PAT_DIRECT_OUT", "0")
+    tuning(direct_out=0)
     g, need = plan(64, 100)
     assert g.num_slots == 1 and need > 0
+
+
+def test_slot_buffer_sizes_without_a_gpu():
+    lib = _lib.load()
+    a = _args()
+    need = C.c_size_t()
+    assert lib.pat_fwd_slots_bytes(C.byref(a), C.byref(need)) == 0
+    # one count per sequence + one ordinal per q_table entry, each piece 256-byte aligned
+    assert need.value == 256 + 256 + 256     # 64 counts, 4 x 16 and 64 x 1 entries
+    offsets = (C.c_int64 * 2)()
+    assert lib.pat_fwd_derive_slots(C.byref(a), None, 0, offsets, None) == _lib.PAT_ERR_INVALID
+    assert lib.pat_fwd_derive_slots(C.byref(a), C.c_void_p(0x10000), 16, offsets, None) == _lib.PAT_ERR_WORKSPACE
+
+def test_tuning_round_trip(tuning):
+    lib = _lib.load()
+    tuning(chunk_tokens=256, direct_out=0)
+    t = _lib.FwdTuning()
+    assert lib.pat_fwd_get_tuning(C.byref(t)) == 0
+    assert (t.chunk_tokens, t.tall_chunk_tokens, t.head_per_wave_tokens, t.direct_out) == (256, 0, -1, 0)
+    g = _lib.FwdGeometry()
+    assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0 and g.chunk_tokens == 256
 
 
 def test_tree_handles_and_errors():

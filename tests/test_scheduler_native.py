@@ -188,3 +188,31 @@ def test_flat_plan_marks_even_buckets():
             assert f == (1 if 4 * int(kv.min()) >= 3 * int(kv.max()) else 0)
     assert flags["c5b"] == [1]          # 32 requests of 4096 tokens
     assert flags["c3"][-1] == 0         # leaves of 128..1024 tokens
+
+
+def test_repeated_pack_keeps_slots_and_box_counts_consistent():
+    # the reference's split counters count on over repeated pack_schedule calls on one tree
+    # (prefix_attn/prefix_tree.py:149 resets them only on a rebuild); the ordinals a launch files
+    # partial results by, and the box counts it merges, describe the current plan alone
+    w = workloads.make("c4", seed=0)
+    t = PrefixTreeCPP(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.padded_table())
+    seen = []
+    for _ in range(2):
+        t.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+        ki = t.kernel_info
+        top = torch.zeros(w.batch, dtype=torch.int64)
+        count = torch.zeros(w.batch, dtype=torch.int64)
+        for q, sl, n in zip(ki.q_tables, ki.slot_tables, ki.num_seqs_per_CTAs):
+            for row in range(q.shape[0]):
+                k = int(n[row])
+                ids, ords = q[row, :k].long(), sl[row, :k].long()
+                top[ids] = torch.maximum(top[ids], ords)
+                count[ids] += 1
+        assert torch.equal(top + 1, ki.num_boxes_per_seq.long())
+        assert torch.equal(count, ki.num_boxes_per_seq.long())
+        assert ki.max_boxes_per_seq == int(count.max())
+        seen.append((ki.num_split_per_seq.clone(), ki.num_boxes_per_seq.clone()))
+    assert torch.equal(seen[0][0], seen[0][1])            # first pack: the two counts agree
+    assert torch.equal(seen[1][0], 2 * seen[0][0])        # second pack: the reference's counter doubled
+    assert torch.equal(seen[1][1], seen[0][1])            # ... the plan's own count did not
