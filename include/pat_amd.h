@@ -293,6 +293,19 @@ int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
  * returns without synchronising. */
 int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
 
+/* pat_fwd_launch for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc). No counterpart in the reference, whose
+ * forward allocates its partial buffers per call (csrc/api.h:217-229). Same arguments, kernels and
+ * results as pat_fwd_launch; args->workspace / workspace_bytes are ignored: the partial results go
+ * to an array built into the library (pat_fwd_static_scratch_bytes() bytes, 64 MiB, one copy per GPU,
+ * held until the process ends). Calls no hipMalloc / hipFree. A launch that needs more partial-result
+ * space than the array holds fails with PAT_ERR_WORKSPACE and enqueues nothing. Every call on a GPU
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls
+ * on one stream are ordered and safe. Nothing in the array has to be cleared between calls: every
+ * slot a call reads it writes first. */
+int pat_fwd_launch_static(const pat_fwd_args* args, void* hip_stream);
+size_t pat_fwd_static_scratch_bytes(void);
+
 /* Partial-result slots for a plan that carries none (pat_fwd_bucket.q_slot == NULL), e.g. the
  * tensors of KernelInfo.to_tensor passed positionally as benchmark/benchmark_kernel.py:247-265
  * does. Filing partial results by CTA_rank, as the reference kernel does

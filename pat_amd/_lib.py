@@ -147,6 +147,8 @@ SYMBOLS = {
     "pat_fwd_validate": (C.c_int, [C.POINTER(FwdArgs)]),
     "pat_fwd_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_launch": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "pat_fwd_launch_static": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p]),
+    "pat_fwd_static_scratch_bytes": (C.c_size_t, []),
     "pat_fwd_slots_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_derive_slots": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_size_t, i64p, C.c_void_p]),
     "pat_fwd_set_tuning": (C.c_int, [C.POINTER(FwdTuning)]),

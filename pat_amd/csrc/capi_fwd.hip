@@ -511,8 +511,15 @@ __global__ void __launch_bounds__(256) pat_slot_kernel(const SlotParams p) {
   if (lane == 0) p.num_boxes_per_seq[s] = count;
 }
 
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+constexpr int kMaxDevices = 64;
+
 }  // namespace
 }  // namespace pat
+
+// Scratch of pat_fwd_launch_static: partial results of one call. One copy per GPU, held until the
+// process ends; host code reaches it only through the address hipGetSymbolAddress returns.
+static __device__ __align__(256) unsigned char scratch[pat::kStaticScratchBytes];
 
 extern "C" {
 
@@ -528,6 +535,42 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
   if (need > 0 && reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
     return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   return launch_core(args, g, args->workspace, hip_stream);
+}
+
+size_t pat_fwd_static_scratch_bytes(void) { return pat::kStaticScratchBytes; }
+
+int pat_fwd_launch_static(const pat_fwd_args* args, void* hip_stream) {
+  using namespace pat;
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  const size_t need = workspace_need(args, g);
+  if (need > kStaticScratchBytes)
+    return fail(PAT_ERR_WORKSPACE, "pat_fwd_launch_static: this launch needs " + std::to_string(need) +
+                                       " bytes of partial results, the built-in scratch holds " +
+                                       std::to_string(kStaticScratchBytes) + "; use pat_fwd_launch with a workspace");
+  // the array's device address, looked up once per device with that device current
+  static std::mutex mutex;
+  static void* device_ptr[kMaxDevices] = {nullptr};
+  int dev = -1;
+  if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(PAT_ERR_INVALID, "pat_fwd_launch_static: device index out of range");
+  void* ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(mutex);
+    if (device_ptr[dev] == nullptr) {
+      void* found = nullptr;
+      if (const hipError_t e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)); e != hipSuccess)
+        return hip_fail(e, "hipGetSymbolAddress(scratch)");
+      if (found == nullptr || reinterpret_cast<uintptr_t>(found) % 256 != 0)
+        return fail(PAT_ERR_HIP, "hipGetSymbolAddress(scratch) returned an unusable address");
+      device_ptr[dev] = found;
+    }
+    ptr = device_ptr[dev];
+  }
+  // Nothing in the scratch has to start at zero: every slot the merge kernel reads is written in
+  // the same call, by the workgroup that fills it or, with -inf, by the one that knows it stays empty.
+  return launch_core(args, g, ptr, hip_stream);
 }
 
 int pat_fwd_slots_bytes(const pat_fwd_args* args, size_t* bytes) {

@@ -163,8 +163,9 @@ def test_single_slot_launch_needs_no_workspace(tuning):
     assert g.num_slots == 1 and need > 0
 
 
-def test_slot_buffer_sizes_without_a_gpu():
+def test_static_scratch_and_slot_buffer_sizes_without_a_gpu():
     lib = _lib.load()
+    assert lib.pat_fwd_static_scratch_bytes() == 64 << 20
     a = _args()
     need = C.c_size_t()
     assert lib.pat_fwd_slots_bytes(C.byref(a), C.byref(need)) == 0
@@ -173,6 +174,12 @@ def test_slot_buffer_sizes_without_a_gpu():
     offsets = (C.c_int64 * 2)()
     assert lib.pat_fwd_derive_slots(C.byref(a), None, 0, offsets, None) == _lib.PAT_ERR_INVALID
     assert lib.pat_fwd_derive_slots(C.byref(a), C.c_void_p(0x10000), 16, offsets, None) == _lib.PAT_ERR_WORKSPACE
+    # a launch whose partial results exceed the built-in scratch is refused before any GPU call
+    big = _args(batch=4096, max_split_per_seq=32)
+    assert lib.pat_fwd_workspace_bytes(C.byref(big), C.byref(need)) == 0 and need.value > (64 << 20)
+    assert lib.pat_fwd_launch_static(C.byref(big), None) == _lib.PAT_ERR_WORKSPACE
+    assert "built-in scratch" in _lib.last_error()
+
 
 def test_tuning_round_trip(tuning):
     lib = _lib.load()

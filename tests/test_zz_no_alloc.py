@@ -1,0 +1,56 @@
+"""The entry point that allocates nothing (pat_fwd_launch_static) against pat_fwd_launch, through
+the C ABI: same kernels, the partial results in the library's built-in scratch array instead of a
+caller's workspace. Two calls in a row, the second on a smaller batch (the scratch keeps the first
+call's contents), bit-identical outputs required."""
+import ctypes as C
+import math
+
+import pytest
+import torch
+
+from pat_amd import PrefixTreeCPP, _lib, _prefix_attn, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _both_routes(name, w, dev):
+    lib = _lib.load()
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    lt = info.launch_tables()
+    results = []
+    for static in (False, True):
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+        L = _prefix_attn._prepare(q, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
+                                  lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
+                                  info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                                  1.0 / math.sqrt(w.head_dim), out, lse, lt["slot_tables"], lt.get("flags"))
+        assert 0 < L.need <= lib.pat_fwd_static_scratch_bytes()
+        stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        if static:
+            L.args.workspace, L.args.workspace_bytes = None, 0
+            rc = lib.pat_fwd_launch_static(C.byref(L.args), stream)
+        else:
+            ws = torch.empty(L.need, dtype=torch.uint8, device=dev)
+            L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), L.need
+            rc = lib.pat_fwd_launch(C.byref(L.args), stream)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        results.append((out, lse))
+    (out_a, lse_a), (out_b, lse_b) = results
+    print(f"[no-alloc] {name}: workspace {L.need} bytes, outputs identical: {torch.equal(out_a, out_b)}", flush=True)
+    assert not torch.isnan(out_b.float()).any() and not torch.isnan(lse_b).any()
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+
+
+def test_static_scratch_entry_point_matches_workspace_entry_point():
+    assert torch.cuda.is_available(), "GPU tests need an AMD GPU"
+    dev = torch.device("cuda:0")
+    print("[case] pat_fwd_launch_static vs pat_fwd_launch: c2, then the smaller c1", flush=True)
+    _both_routes("c2", workloads.make("c2", seed=0), dev)
+    _both_routes("c1", workloads.make("c1", seed=0), dev)   # smaller: stale partial results stay behind it
