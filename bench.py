@@ -93,7 +93,7 @@ def main() -> None:
         sys.exit(2)
 
     import torch
-    from pat_amd import PrefixTreeCPP, _lib, _prefix_attn, workloads
+    from pat_amd import PrefixTreeCPP, _ctypes_launch, _lib, workloads
 
     assert torch.cuda.is_available(), "bench.py needs an AMD GPU"
     dev = torch.device("cuda:0")
@@ -130,7 +130,7 @@ def main() -> None:
     def prepare(plan_kw, slots):
         launches = []
         for i in range(copies):
-            L = _prefix_attn._prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
+            L = _ctypes_launch.prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
                                       plan_kw["block_tables"], plan_kw["num_seqs_per_CTAs"], plan_kw["CTA_ranks"],
                                       plan_kw["kv_in_CTAs"], plan_kw["MNW"], plan_kw["max_split_per_seq"],
                                       plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots,

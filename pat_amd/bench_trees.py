@@ -40,7 +40,7 @@ def unique_tokens(spec: str) -> int:
 
 
 def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budget_bytes: int) -> dict:
-    from . import PrefixTreeCPP, _lib, _prefix_attn, generate_tree_seqs, workloads
+    from . import PrefixTreeCPP, _ctypes_launch, _lib, generate_tree_seqs, workloads
 
     dev = torch.device("cuda:0")
     lib = _lib.load()
@@ -71,7 +71,7 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
     oblivious = workloads.oblivious_plan(w, dev)
 
     def launches(plan, slots):
-        made = [_prefix_attn._prepare(q, ks[i], vs[i], plan["num_split_per_seq"], plan["query_tables"],
+        made = [_ctypes_launch.prepare(q, ks[i], vs[i], plan["num_split_per_seq"], plan["query_tables"],
                                       plan["block_tables"], plan["num_seqs_per_CTAs"], plan["CTA_ranks"],
                                       plan["kv_in_CTAs"], plan["MNW"], plan["max_split_per_seq"],
                                       plan["max_seqs_in_CTA"], plan["max_blocks_in_CTA"], scale, out, None, slots,

@@ -1,11 +1,14 @@
-"""Builds pat_amd/libpat_amd.so in-tree with hipcc for gfx950 (MI355X).
+"""Builds pat_amd/libpat_amd.so and the PyTorch-ROCm extension pat_amd/_prefix_attn.so in-tree.
 
-    python -m pat_amd.build            # compile every source, link the library
+    python -m pat_amd.build            # compile every source, link both
     python -m pat_amd.build --jobs 4   # parallel compile
 
-hipcc cross-compiles gfx950 code objects without a GPU, so this runs on any ROCm
-host. The scheduler sources are plain C++17 and are compiled by the same driver so
-that one shared object carries the whole C ABI of include/pat_amd.h.
+libpat_amd.so: hipcc, gfx950 (MI355X). hipcc cross-compiles gfx950 code objects without a GPU,
+so this runs on any ROCm host. The scheduler sources are plain C++17 and are compiled by the same
+driver so that one shared object carries the whole C ABI of include/pat_amd.h.
+
+_prefix_attn.so: the pybind11 / libtorch binding over that C ABI (host code only, g++), linked
+against libpat_amd.so (found through its own directory at run time) and the installed torch.
 """
 from __future__ import annotations
 
@@ -81,12 +84,51 @@ def build(jobs: int = 4, verbose: bool = False) -> str:
     return OUT
 
 
+EXT_SRC = os.path.join(CSRC, "torch_ext", "prefix_attn_ext.cc")
+EXT_OUT = os.path.join(HERE, "_prefix_attn.so")
+
+
+def build_extension(verbose: bool = False) -> str:
+    """Compiles the torch binding (one translation unit, about a minute) and links it."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("g++ not found: needed for the torch extension")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    includes = [os.path.join(ROOT, "include"), *ce.include_paths(), os.path.join(rocm, "include"),
+                sysconfig.get_paths()["include"]]
+    abi = int(bool(torch._C._GLIBCXX_USE_CXX11_ABI))
+    tmp = EXT_OUT + ".tmp"
+    cmd = [cxx, "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wno-unused-parameter", "-Wno-sign-compare",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+           "-DTORCH_EXTENSION_NAME=_prefix_attn", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           *[f"-isystem{p}" if "torch" in p or "rocm" in p else f"-I{p}" for p in includes],
+           EXT_SRC, "-o", tmp,
+           f"-L{HERE}", "-lpat_amd", f"-L{torch_lib}", "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+           "-lc10", "-lc10_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building the torch extension failed:\n{res.stderr[-4000:]}")
+    os.replace(tmp, EXT_OUT)
+    return EXT_OUT
+
+
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--jobs", type=int, default=4)
     ap.add_argument("-v", "--verbose", action="store_true")
+    ap.add_argument("--no-extension", action="store_true", help="only libpat_amd.so (seconds), not the torch binding")
     a = ap.parse_args()
+    ap_ext = not a.no_extension
     print(build(a.jobs, a.verbose))
+    if ap_ext:
+        print(build_extension(a.verbose))
 
 
 if __name__ == "__main__":

@@ -1,0 +1,641 @@
+// The compiled PyTorch-ROCm extension `_prefix_attn`: the Python surface of the reference's
+// extension module (csrc/bindings.cpp:74-158 of the flashserve/PAT tree) over the C ABI of
+// libpat_amd (include/pat_amd.h). Host code only: no kernel lives here. torch supplies device
+// pointers, strides, the current HIP stream and scratch memory from its caching allocator.
+//
+//   prefix_attn_with_kvcache   table overload (bindings.cpp:7-43, :76-95) and tree overload
+//                              (:45-72, :148-157)
+//   PrefixTreeCPP              build_radix_tree / pack_schedule with the GIL released
+//                              (:100-146), kernel_info
+//   KernelInfo                 plan tensors + to_gpu (:97-98; csrc/prefix_tree.h:7-39)
+//   paged_decode_baseline      the prefix-oblivious comparator (not in the reference's API)
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "pat_amd.h"
+
+namespace py = pybind11;
+
+namespace {
+
+using TensorList = std::vector<at::Tensor>;
+
+// ---- errors ---------------------------------------------------------------------------------
+// PAT_ERR_* -> the exception the reference API raises in the same situation. Call with the GIL held.
+void check(int code) {
+  if (code == PAT_OK) return;
+  const std::string msg = pat_last_error();
+  switch (code) {
+    case PAT_ERR_VALUE:
+      if (msg.find("by zero") != std::string::npos) {
+        PyErr_SetString(PyExc_ZeroDivisionError, msg.c_str());
+        throw py::error_already_set();
+      }
+      throw py::value_error(msg);
+    case PAT_ERR_INDEX: throw py::index_error(msg);
+    case PAT_ERR_KEY: throw py::key_error(msg);
+    default: throw std::runtime_error(msg);
+  }
+}
+
+void require(bool cond, const char* msg) {
+  if (!cond) throw std::runtime_error(msg);
+}
+void require(bool cond, const std::string& msg) {
+  if (!cond) throw std::runtime_error(msg);
+}
+
+void* raw_stream(const c10::Device& dev) {
+  return static_cast<void*>(c10::hip::getCurrentHIPStream(dev.index()).stream());
+}
+
+c10::Device to_device(const py::object& obj) {
+  if (py::isinstance<py::str>(obj)) return c10::Device(obj.cast<std::string>());
+  return obj.cast<c10::Device>();
+}
+
+// ---- a prepared launch ------------------------------------------------------------------------
+// pat_fwd_args plus everything it points into. Built once per set of tensors (a decode step calls
+// the forward once per layer with the same plan), launched many times.
+struct Prepared {
+  pat_fwd_args args;
+  std::vector<pat_fwd_bucket> buckets;
+  TensorList keep;          // plan tensors (and derived slots) stay alive as long as the launch does
+  size_t need = 0;          // workspace bytes
+  Prepared() { std::memset(&args, 0, sizeof(args)); }
+};
+
+void strides3(const at::Tensor& t, int64_t out[3]) {
+  out[0] = t.stride(0); out[1] = t.stride(1); out[2] = t.stride(2);
+}
+
+struct PlanTables {
+  const TensorList* q_tables;
+  const TensorList* block_tables;
+  const TensorList* num_seqs;
+  const TensorList* ranks;
+  const TensorList* kvs;
+  const TensorList* slots;                       // may be null
+  const std::vector<std::vector<int>>* mnw;
+  const std::vector<int>* flags;                 // may be null
+};
+
+// Checks that need tensor metadata follow csrc/api.h:131-181, :256-277 of the reference.
+std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                                  const at::Tensor& num_split, const PlanTables& pt, int max_split, int max_seqs,
+                                  int max_blocks, double scale, const at::Tensor& out,
+                                  const std::optional<at::Tensor>& lse) {
+  require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "only support fp16 and bf16 data type");
+  require(k.scalar_type() == q.scalar_type(), "query and key must have the same dtype");
+  require(v.scalar_type() == q.scalar_type(), "query and value must have the same dtype");
+  require(q.is_cuda(), "q must be on CUDA");
+  require(k.is_cuda(), "kcache must be on CUDA");
+  require(v.is_cuda(), "vcache must be on CUDA");
+  for (const at::Tensor* t : {&q, &k, &v})
+    require(t->dim() == 4 && t->stride(-1) == 1, "Input tensor must have contiguous last dimension");
+  const int64_t b = q.size(0), sq = q.size(1), h = q.size(2), d = q.size(3);
+  const int64_t nblk = k.size(0), page = k.size(1), hk = k.size(2);
+  require(k.size(3) == d, "kcache must have shape (num_blocks, page_block_size, n_heads_kv, head_size_og)");
+  require(v.sizes() == k.sizes(), "vcache must have shape (num_blocks, page_block_size, n_heads_kv, head_size_og)");
+  require(out.is_cuda() && out.scalar_type() == q.scalar_type() && out.sizes() == q.sizes() && out.stride(-1) == 1,
+          "out must be a CUDA tensor with q's shape and dtype and a contiguous last dimension");
+  require(num_split.is_cuda(), "num_split_per_seq must be on CUDA");
+  require(num_split.scalar_type() == at::kInt, "num_split_per_seq must have dtype torch.int32");
+  require(num_split.dim() == 1 && num_split.size(0) == b, "num_split_per_seq must have shape (batch_size)");
+  require(num_split.stride(-1) == 1, "num_split_per_seq must have contiguous last dimension");
+  const size_t nb = pt.mnw->size();
+  require(pt.q_tables->size() == nb && pt.block_tables->size() == nb && pt.num_seqs->size() == nb &&
+              pt.ranks->size() == nb && pt.kvs->size() == nb,
+          "MNW and the per-bucket plan lists must have the same length");
+  const TensorList* slots = (pt.slots != nullptr && !pt.slots->empty()) ? pt.slots : nullptr;
+  require(slots == nullptr || slots->size() == nb, "slot_tables must have one entry per bucket");
+  require(pt.flags == nullptr || pt.flags->empty() || pt.flags->size() == nb, "bucket_flags must have one entry per bucket");
+
+  auto L = std::make_shared<Prepared>();
+  L->buckets.resize(std::max<size_t>(nb, 1));
+  std::memset(L->buckets.data(), 0, L->buckets.size() * sizeof(pat_fwd_bucket));
+  for (size_t i = 0; i < nb; ++i) {
+    const at::Tensor &qt = (*pt.q_tables)[i], &bt = (*pt.block_tables)[i], &ns = (*pt.num_seqs)[i],
+                     &rk = (*pt.ranks)[i], &kv = (*pt.kvs)[i];
+    const std::pair<const char*, const at::Tensor*> named[] = {
+        {"query_tables", &qt}, {"block_tables", &bt}, {"num_seqs_per_CTA", &ns}, {"CTA_rank", &rk}, {"kv_in_CTA", &kv}};
+    for (const auto& nt : named) {
+      require(nt.second->is_cuda(), std::string(nt.first) + " must be on CUDA");
+      require(nt.second->scalar_type() == at::kInt, std::string(nt.first) + " must have dtype torch.int32");
+      require(nt.second->numel() == 0 || nt.second->stride(-1) == 1,
+              std::string(nt.first) + " must have contiguous last dimension");
+    }
+    require(qt.dim() == 2 && bt.dim() == 2 && bt.size(0) == qt.size(0), "query_tables / block_tables must be (CTAs, width)");
+    const int64_t ctas = qt.size(0);
+    for (int j = 2; j < 5; ++j)
+      require(named[j].second->dim() == 1 && named[j].second->size(0) == ctas,
+              std::string(named[j].first) + " must have shape (CTAs)");
+    pat_fwd_bucket& fb = L->buckets[i];
+    fb.q_table = qt.data_ptr<int32_t>(); fb.block_table = bt.data_ptr<int32_t>();
+    fb.num_seqs = ns.data_ptr<int32_t>(); fb.rank = rk.data_ptr<int32_t>(); fb.kv = kv.data_ptr<int32_t>();
+    if (slots != nullptr) {
+      const at::Tensor& st = (*slots)[i];
+      require(st.is_cuda() && st.scalar_type() == at::kInt && st.sizes() == qt.sizes() && st.strides() == qt.strides(),
+              "slot_tables must match query_tables (CUDA int32, same layout)");
+      fb.q_slot = st.data_ptr<int32_t>();
+      L->keep.push_back(st);
+    }
+    fb.q_table_stride = ctas > 1 ? qt.stride(0) : std::max<int64_t>(qt.size(1), 1);
+    fb.block_table_stride = ctas > 1 ? bt.stride(0) : std::max<int64_t>(bt.size(1), 1);
+    fb.num_boxes = (int32_t)ctas; fb.max_seqs = (int32_t)qt.size(1); fb.max_blocks = (int32_t)bt.size(1);
+    require((*pt.mnw)[i].size() == 3, "MNW entries must be [M, N, W]");
+    for (int j = 0; j < 3; ++j) fb.mnw[j] = (*pt.mnw)[i][(size_t)j];
+    fb.flags = (pt.flags != nullptr && !pt.flags->empty()) ? (*pt.flags)[i] : 0;
+    for (const auto& nt : named) L->keep.push_back(*nt.second);
+  }
+  L->keep.push_back(num_split);
+
+  pat_fwd_args& a = L->args;
+  a.dtype = q.scalar_type() == at::kBFloat16 ? PAT_DTYPE_BF16 : PAT_DTYPE_F16;
+  a.batch = (int32_t)b; a.seqlen_q = (int32_t)sq; a.heads = (int32_t)h; a.kv_heads = (int32_t)hk;
+  a.head_dim = (int32_t)d; a.page_size = (int32_t)page; a.num_pages = (int32_t)nblk;
+  a.q = q.data_ptr(); a.k = k.data_ptr(); a.v = v.data_ptr(); a.out = out.data_ptr();
+  strides3(q, a.q_stride); strides3(k, a.k_stride); strides3(v, a.v_stride); strides3(out, a.o_stride);
+  a.num_split_per_seq = num_split.data_ptr<int32_t>();
+  a.max_split_per_seq = max_split; a.max_seqs_in_box = max_seqs; a.max_blocks_in_box = max_blocks;
+  a.softmax_scale = (float)scale;
+  a.num_buckets = (int32_t)nb;
+  a.buckets = L->buckets.data();
+  if (lse.has_value()) {
+    require(lse->is_cuda() && lse->scalar_type() == at::kFloat && lse->is_contiguous() && lse->numel() == b * h,
+            "softmax_lse must be a contiguous CUDA float32 tensor with batch_size * n_heads elements");
+    a.lse_out = lse->data_ptr<float>();
+  }
+  if (slots == nullptr && max_split > 1) {
+    // A plan without slot tables (the reference's call form): CTA_rank is not unique per sequence on
+    // irregular forests, so the ordinals are derived from the q_tables on the device, once per
+    // prepared launch (the caches key on the tables' version counters).
+    size_t sbytes = 0;
+    check(pat_fwd_slots_bytes(&a, &sbytes));
+    at::Tensor derived = at::empty({(int64_t)sbytes}, at::TensorOptions().dtype(at::kByte).device(q.device()));
+    std::vector<int64_t> offsets(std::max<size_t>(nb, 1), 0);
+    check(pat_fwd_derive_slots(&a, derived.data_ptr(), sbytes, offsets.data(), raw_stream(q.device())));
+    int32_t* base = static_cast<int32_t*>(derived.data_ptr());
+    for (size_t i = 0; i < nb; ++i) L->buckets[i].q_slot = base + offsets[i];
+    a.num_split_per_seq = base;
+    L->keep.push_back(derived);
+  }
+  check(pat_fwd_workspace_bytes(&a, &L->need));
+  return L;
+}
+
+void run(Prepared& L, const c10::Device& dev) {
+  at::Tensor ws;   // scratch for the partial results (none for a single-slot launch); stream-ordered reuse
+  if (L.need > 0) {
+    ws = at::empty({(int64_t)L.need}, at::TensorOptions().dtype(at::kByte).device(dev));
+    L.args.workspace = ws.data_ptr();
+  } else {
+    L.args.workspace = nullptr;
+  }
+  L.args.workspace_bytes = L.need;
+  check(pat_fwd_launch(&L.args, raw_stream(dev)));
+}
+
+// ---- cache keys -----------------------------------------------------------------------------------
+struct Key {
+  std::string bytes;
+  template <typename T> void add(const T& v) { bytes.append(reinterpret_cast<const char*>(&v), sizeof(T)); }
+  void tensor(const at::Tensor& t) {   // address + layout
+    add(t.data_ptr()); add((int)t.scalar_type()); add((int64_t)t.dim());
+    for (int64_t s : t.sizes()) add(s);
+    for (int64_t s : t.strides()) add(s);
+  }
+  void plan_tensor(const at::Tensor& t) {   // ... and the version counter: in-place edits of a plan count
+    tensor(t); add((int64_t)t._version());
+  }
+};
+
+// ---- KernelInfo -----------------------------------------------------------------------------------
+struct LaunchPart { int bucket, lo, hi; };
+
+struct KernelInfo {
+  TensorList q_tables, block_tables, num_seqs, ranks, kvs, slot_tables;
+  std::vector<std::vector<int>> mnws;
+  at::Tensor num_split_per_seq = at::empty({0}, at::kInt);
+  at::Tensor num_boxes_per_seq = at::empty({0}, at::kInt);
+  int max_split = 0, max_boxes = 0, max_seqs = 0, max_blocks = 0;
+  // launch copies: every bucket's boxes longest first, a bucket with a wide head split in two
+  bool has_launch = false;
+  TensorList l_q_tables, l_block_tables, l_num_seqs, l_ranks, l_kvs, l_slot_tables;
+  std::vector<std::vector<int>> l_mnws;
+  std::vector<int> l_flags;
+  TensorList launch_order;                          // per bucket: launch position -> scheduler row
+  std::vector<std::vector<LaunchPart>> launch_parts;  // per bucket: its launch buckets
+  // the whole plan in one int32 buffer (pinned on the host when a GPU is there)
+  std::optional<at::Tensor> flat;
+  pat_flat_plan layout;
+  std::unordered_map<std::string, std::shared_ptr<Prepared>> cache;
+
+  void clear_tables() {
+    for (TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables, &l_q_tables,
+                          &l_block_tables, &l_num_seqs, &l_ranks, &l_kvs, &l_slot_tables, &launch_order})
+      l->clear();
+    mnws.clear(); l_mnws.clear(); l_flags.clear(); launch_parts.clear();
+    cache.clear();
+  }
+
+  // (Re)creates every plan tensor as a view of `buf` (the host buffer or its copy on a device).
+  void bind(const at::Tensor& buf) {
+    clear_tables();
+    const pat_flat_plan& lay = layout;
+    auto vec = [&](int64_t off, int64_t n) { return buf.narrow(0, off, n); };
+    auto mat = [&](int64_t off, int64_t n, int64_t w) { return buf.narrow(0, off, n * w).view({n, w}); };
+    num_split_per_seq = vec(lay.num_split_per_seq, lay.batch);
+    num_boxes_per_seq = vec(lay.num_boxes_per_seq, lay.batch);
+    for (int b = 0; b < lay.num_buckets; ++b) {
+      const pat_flat_bucket& f = lay.buckets[b];
+      mnws.push_back({f.mnw[0], f.mnw[1], f.mnw[2]});
+      q_tables.push_back(mat(f.q_table, f.num_boxes, f.max_seqs));
+      slot_tables.push_back(mat(f.q_slot, f.num_boxes, f.max_seqs));
+      block_tables.push_back(mat(f.block_table, f.num_boxes, f.max_blocks));
+      num_seqs.push_back(vec(f.num_seqs, f.num_boxes));
+      ranks.push_back(vec(f.rank, f.num_boxes));
+      kvs.push_back(vec(f.kv, f.num_boxes));
+      launch_order.push_back(vec(lay.launch_order[b], f.num_boxes));
+      launch_parts.emplace_back();
+    }
+    for (int i = 0; i < lay.num_launch_buckets; ++i) {
+      const pat_flat_bucket& f = lay.launch[i];
+      l_mnws.push_back({f.mnw[0], f.mnw[1], f.mnw[2]});
+      l_flags.push_back(f.flags);
+      l_q_tables.push_back(mat(f.q_table, f.num_boxes, f.max_seqs));
+      l_slot_tables.push_back(mat(f.q_slot, f.num_boxes, f.max_seqs));
+      l_block_tables.push_back(mat(f.block_table, f.num_boxes, f.max_blocks));
+      l_num_seqs.push_back(vec(f.num_seqs, f.num_boxes));
+      l_ranks.push_back(vec(f.rank, f.num_boxes));
+      l_kvs.push_back(vec(f.kv, f.num_boxes));
+      launch_parts[(size_t)f.parent].push_back({i, f.first, f.first + f.num_boxes});
+    }
+    has_launch = true;
+  }
+
+  // Copies every plan tensor to `device`: one copy of the one buffer, asynchronous from pinned memory
+  // (the reference moves each table by itself, csrc/prefix_tree.h:27-38).
+  void to_gpu(const c10::Device& device) {
+    if (flat.has_value()) {
+      flat = flat->to(device, /*non_blocking=*/true);
+      bind(*flat);
+      return;
+    }
+    auto move = [&](TensorList& l) { for (auto& t : l) t = t.to(device, true); };
+    for (TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables}) move(*l);
+    num_split_per_seq = num_split_per_seq.to(device, true);
+    num_boxes_per_seq = num_boxes_per_seq.to(device, true);
+    cache.clear();
+  }
+
+  py::dict launch_tables() const {
+    py::dict d;
+    const bool l = has_launch;
+    d["q_tables"] = l ? l_q_tables : q_tables;
+    d["slot_tables"] = l ? l_slot_tables : slot_tables;
+    d["block_tables"] = l ? l_block_tables : block_tables;
+    d["num_seqs_per_CTAs"] = l ? l_num_seqs : num_seqs;
+    d["CTA_ranks"] = l ? l_ranks : ranks;
+    d["kv_in_CTAs"] = l ? l_kvs : kvs;
+    d["MNWs"] = l ? l_mnws : mnws;
+    d["flags"] = l ? l_flags : std::vector<int>(mnws.size(), 0);
+    return d;
+  }
+
+  // For the boxes of scheduler bucket b, in scheduler order: (launch bucket, row in it).
+  std::pair<at::Tensor, at::Tensor> launch_position(int b) const {
+    require(b >= 0 && (size_t)b < launch_order.size(), "bucket index out of range");
+    const at::Tensor order = launch_order[(size_t)b].to(at::kCPU).to(at::kLong).contiguous();
+    const int64_t n = order.numel();
+    at::Tensor bucket = at::empty({n}, at::kLong), row = at::empty({n}, at::kLong);
+    const int64_t* o = order.data_ptr<int64_t>();
+    int64_t* pb = bucket.data_ptr<int64_t>();
+    int64_t* pr = row.data_ptr<int64_t>();
+    for (const LaunchPart& p : launch_parts[(size_t)b])
+      for (int64_t pos = p.lo; pos < p.hi; ++pos) { pb[o[pos]] = p.bucket; pr[o[pos]] = pos - p.lo; }
+    return {bucket, row};
+  }
+};
+
+at::Tensor host_i32(int64_t n, const int32_t* src) {
+  at::Tensor t = at::empty({n}, at::kInt);
+  if (n > 0) std::memcpy(t.data_ptr<int32_t>(), src, (size_t)n * sizeof(int32_t));
+  return t;
+}
+
+// ---- PrefixTreeCPP ----------------------------------------------------------------------------------
+struct TreeHandle {
+  pat_tree* h = nullptr;
+  ~TreeHandle() { if (h) pat_tree_destroy(h); }
+};
+
+struct PrefixTreeCPP {
+  int block_size;
+  std::shared_ptr<TreeHandle> native = std::make_shared<TreeHandle>();
+  std::shared_ptr<KernelInfo> info = std::make_shared<KernelInfo>();
+
+  explicit PrefixTreeCPP(int bs) : block_size(bs) { check(pat_tree_create(bs, &native->h)); }
+
+  void build_radix_tree(const py::object& seq_lens, const py::object& table_obj) {
+    require(THPVariable_Check(table_obj.ptr()), "block_table must be a 2-D CPU Int32 Tensor");
+    const at::Tensor table_in = table_obj.cast<at::Tensor>();
+    require(table_in.dim() == 2, "block_table must be a 2-D CPU Int32 Tensor");
+    require(table_in.device().is_cpu() && table_in.scalar_type() == at::kInt, "block_table must be a CPU Int32 Tensor");
+    const at::Tensor table = table_in.contiguous();
+    std::vector<int32_t> lens_vec;
+    at::Tensor lens_t;
+    const int32_t* lens = nullptr;
+    int64_t n_lens = 0;
+    if (THPVariable_Check(seq_lens.ptr())) {
+      lens_t = seq_lens.cast<at::Tensor>();
+      require(lens_t.device().is_cpu() && lens_t.scalar_type() == at::kInt,
+              "seq_lens must be a List[int] or a CPU Int32 Tensor");
+      lens_t = lens_t.reshape({-1}).contiguous();
+      lens = lens_t.data_ptr<int32_t>(); n_lens = lens_t.numel();
+    } else if (py::isinstance<py::list>(seq_lens)) {
+      lens_vec = seq_lens.cast<std::vector<int32_t>>();
+      lens = lens_vec.data(); n_lens = (int64_t)lens_vec.size();
+    } else {
+      throw std::runtime_error("seq_lens must be a List[int] or a CPU Int32 Tensor");
+    }
+    require(n_lens == table.size(0), "Seq lens list mismatch");
+    int rc;
+    {
+      py::gil_scoped_release release;   // the tree is built without the GIL (csrc/bindings.cpp:124)
+      rc = pat_tree_build(native->h, lens, table.data_ptr<int32_t>(), (int32_t)table.size(0), (int32_t)table.size(1));
+    }
+    check(rc);
+  }
+
+  void pack_schedule(const py::object& mnws_obj, int hratio, int kv_head, bool use_compute_model) {
+    std::vector<int32_t> mnws;
+    bool given = false;
+    if (!mnws_obj.is_none()) {
+      const auto rows = mnws_obj.cast<std::vector<std::vector<int>>>();
+      // an empty list selects the default buckets (csrc/prefix_tree.h:189)
+      for (const auto& r : rows) {
+        require(r.size() == 3, "MNWs entries must be [M, N, W]");
+        mnws.insert(mnws.end(), r.begin(), r.end());
+      }
+      given = !rows.empty();
+    }
+    auto fresh = std::make_shared<KernelInfo>();
+    int rc, rc_flat = PAT_OK;
+    at::Tensor host;
+    {
+      py::gil_scoped_release release;   // planning runs without the GIL (csrc/bindings.cpp:138)
+      rc = pat_tree_pack(native->h, given ? mnws.data() : nullptr, given ? (int32_t)(mnws.size() / 3) : 0, hratio,
+                         kv_head, use_compute_model ? 1 : 0, nullptr);
+      if (rc == PAT_OK) rc_flat = pat_tree_flat_plan(native->h, &fresh->layout, nullptr, 0);
+    }
+    check(rc);
+    if (rc_flat == PAT_OK) {
+      const int64_t total = std::max<int64_t>(fresh->layout.total, 1);
+      host = at::empty({total}, at::TensorOptions().dtype(at::kInt).pinned_memory(at::hasHIP() || at::hasCUDA()));
+      {
+        py::gil_scoped_release release;
+        rc = pat_tree_flat_plan(native->h, &fresh->layout, host.data_ptr<int32_t>(), host.numel());
+      }
+      check(rc);
+      fresh->flat = host;
+      fresh->max_split = fresh->layout.max_split_per_seq;
+      fresh->max_boxes = fresh->layout.max_boxes_per_seq;
+      fresh->max_seqs = fresh->layout.max_seqs_in_box;
+      fresh->max_blocks = fresh->layout.max_blocks_in_box;
+      fresh->bind(host);
+    } else {
+      // more buckets than one launch takes: the plan can still be read, table by table
+      pat_plan_view view;
+      check(pat_tree_plan(native->h, &view));
+      for (int b = 0; b < view.num_buckets; ++b) {
+        const pat_bucket_view& bk = view.buckets[b];
+        const int64_t n = bk.num_boxes;
+        fresh->mnws.push_back({bk.mnw[0], bk.mnw[1], bk.mnw[2]});
+        fresh->q_tables.push_back(host_i32(n * bk.max_seqs, bk.q_table).view({n, bk.max_seqs}));
+        fresh->slot_tables.push_back(host_i32(n * bk.max_seqs, bk.q_slot).view({n, bk.max_seqs}));
+        fresh->block_tables.push_back(host_i32(n * bk.max_blocks, bk.block_table).view({n, bk.max_blocks}));
+        fresh->num_seqs.push_back(host_i32(n, bk.num_seqs));
+        fresh->ranks.push_back(host_i32(n, bk.rank));
+        fresh->kvs.push_back(host_i32(n, bk.kv));
+      }
+      fresh->num_split_per_seq = host_i32(view.batch, view.num_split_per_seq);
+      fresh->num_boxes_per_seq = host_i32(view.batch, view.num_boxes_per_seq);
+      fresh->max_split = view.max_split_per_seq; fresh->max_boxes = view.max_boxes_per_seq;
+      fresh->max_seqs = view.max_seqs_in_box; fresh->max_blocks = view.max_blocks_in_box;
+    }
+    info = fresh;
+  }
+};
+
+// ---- forward ------------------------------------------------------------------------------------------
+std::mutex g_table_mutex;
+std::unordered_map<std::string, std::shared_ptr<Prepared>> g_table_launches;
+
+struct DeviceScope {   // the kernels launch on the current HIP device: switch only when q lives elsewhere
+  std::optional<c10::DeviceGuard> guard;
+  explicit DeviceScope(const at::Tensor& q) {
+    require(q.is_cuda(), "q must be on CUDA");
+    guard.emplace(q.device());
+  }
+};
+
+void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& num_split,
+                const TensorList& q_tables, const TensorList& block_tables, const TensorList& num_seqs,
+                const TensorList& ranks, const TensorList& kvs, const std::vector<std::vector<int>>& mnw,
+                int max_split, int max_seqs, int max_blocks, double scale, const at::Tensor& out,
+                const py::object& /*timing_: accepted and ignored, the reference never reads it (csrc/api.h:288-290)*/,
+                const std::optional<at::Tensor>& lse, const std::optional<TensorList>& slot_tables,
+                const std::optional<std::vector<int>>& bucket_flags) {
+  require(k.is_cuda(), "kcache must be on CUDA");
+  require(v.is_cuda(), "vcache must be on CUDA");
+  DeviceScope scope(q);
+  // The prepared launch is kept per set of tensors: a decode step calls this once per layer with the
+  // same plan. The key holds what the argument block was built from (addresses, layouts, version
+  // counters of the plan tensors); the tensors' contents are read by the kernels at every call.
+  Key key;
+  key.tensor(q); key.tensor(k); key.tensor(v); key.tensor(out);
+  key.add(lse.has_value()); if (lse.has_value()) key.tensor(*lse);
+  key.plan_tensor(num_split);
+  for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs}) {
+    key.add((int64_t)l->size());
+    for (const at::Tensor& t : *l) key.plan_tensor(t);
+  }
+  for (const auto& m : mnw) for (int x : m) key.add(x);
+  key.add(max_split); key.add(max_seqs); key.add(max_blocks); key.add(scale);
+  key.add(slot_tables.has_value());
+  if (slot_tables.has_value()) for (const at::Tensor& t : *slot_tables) key.plan_tensor(t);
+  if (bucket_flags.has_value()) for (int f : *bucket_flags) key.add(f);
+
+  std::shared_ptr<Prepared> L;
+  {
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    auto it = g_table_launches.find(key.bytes);
+    if (it != g_table_launches.end()) L = it->second;
+  }
+  if (!L) {
+    PlanTables pt{&q_tables, &block_tables, &num_seqs, &ranks, &kvs,
+                  slot_tables.has_value() ? &*slot_tables : nullptr, &mnw,
+                  bucket_flags.has_value() ? &*bucket_flags : nullptr};
+    L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse);
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    if (g_table_launches.size() >= 64) g_table_launches.clear();
+    g_table_launches[key.bytes] = L;
+  }
+  run(*L, q.device());
+}
+
+void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, PrefixTreeCPP& tree, double scale,
+              const at::Tensor& out, const std::optional<at::Tensor>& lse) {
+  require(k.is_cuda(), "kcache must be on CUDA");
+  require(v.is_cuda(), "vcache must be on CUDA");
+  DeviceScope scope(q);
+  KernelInfo& info = *tree.info;
+  Key key;
+  key.tensor(q); key.tensor(k); key.tensor(v); key.tensor(out); key.add(scale);
+  key.add(lse.has_value()); if (lse.has_value()) key.tensor(*lse);
+  std::shared_ptr<Prepared> L;
+  auto it = info.cache.find(key.bytes);
+  if (it != info.cache.end()) {
+    L = it->second;
+  } else {
+    const bool l = info.has_launch;
+    const std::vector<int> no_flags;
+    // partial results are filed by slot_tables: the launch merges each sequence's boxes of THIS plan
+    // (num_split_per_seq counts on over repeated pack_schedule calls)
+    PlanTables pt{l ? &info.l_q_tables : &info.q_tables, l ? &info.l_block_tables : &info.block_tables,
+                  l ? &info.l_num_seqs : &info.num_seqs, l ? &info.l_ranks : &info.ranks, l ? &info.l_kvs : &info.kvs,
+                  l ? &info.l_slot_tables : &info.slot_tables, l ? &info.l_mnws : &info.mnws,
+                  l ? &info.l_flags : &no_flags};
+    require(!pt.mnw->empty(), "the tree has no plan: call pack_schedule and kernel_info.to_gpu first");
+    L = prepare(q, k, v, info.num_boxes_per_seq, pt, info.max_boxes, info.max_seqs, info.max_blocks, scale, out, lse);
+    if (info.cache.size() >= 256) info.cache.clear();
+    info.cache[key.bytes] = L;
+  }
+  run(*L, q.device());
+}
+
+void paged_decode_baseline(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& block_table,
+                           const at::Tensor& seq_lens, double scale, const at::Tensor& out,
+                           const std::optional<at::Tensor>& lse, bool even_lengths) {
+  const std::pair<const char*, const at::Tensor*> named[] = {
+      {"q", &q}, {"kcache", &k}, {"vcache", &v}, {"block_table", &block_table}, {"seq_lens", &seq_lens}};
+  for (const auto& nt : named) require(nt.second->is_cuda(), std::string(nt.first) + " must be on CUDA");
+  require((q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16) && k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type(), "only support fp16 and bf16 data type");
+  require(q.dim() == 4 && k.dim() == 4 && v.dim() == 4, "q, kcache, vcache must be 4-D");
+  require(block_table.scalar_type() == at::kInt && block_table.dim() == 2 && block_table.stride(1) == 1,
+          "block_table must be a 2-D int32 tensor with contiguous rows");
+  require(seq_lens.scalar_type() == at::kInt && seq_lens.dim() == 1 && seq_lens.is_contiguous(),
+          "seq_lens must be a contiguous 1-D int32 tensor");
+  const int64_t b = q.size(0), h = q.size(2), d = q.size(3);
+  require(q.size(1) == 1, "q must have shape (batch_size, 1, n_heads, head_size): decode only");
+  require(block_table.size(0) == b && seq_lens.size(0) == b, "block_table / seq_lens must have one row per request");
+  require(out.is_cuda() && out.scalar_type() == q.scalar_type() && out.sizes() == q.sizes() && out.stride(-1) == 1,
+          "out must be a CUDA tensor with q's shape and dtype and a contiguous last dimension");
+  pat_baseline_args a;
+  std::memset(&a, 0, sizeof(a));
+  a.dtype = q.scalar_type() == at::kBFloat16 ? PAT_DTYPE_BF16 : PAT_DTYPE_F16;
+  a.batch = (int32_t)b; a.heads = (int32_t)h; a.kv_heads = (int32_t)k.size(2); a.head_dim = (int32_t)d;
+  a.page_size = (int32_t)k.size(1); a.num_pages = (int32_t)k.size(0); a.max_blocks = (int32_t)block_table.size(1);
+  a.q = q.data_ptr(); a.k = k.data_ptr(); a.v = v.data_ptr(); a.out = out.data_ptr();
+  strides3(q, a.q_stride); strides3(k, a.k_stride); strides3(v, a.v_stride); strides3(out, a.o_stride);
+  a.block_table = block_table.data_ptr<int32_t>(); a.block_table_stride = block_table.stride(0);
+  a.seq_lens = seq_lens.data_ptr<int32_t>();
+  a.softmax_scale = (float)scale;
+  a.flags = even_lengths ? PAT_BUCKET_EVEN : 0;
+  if (lse.has_value()) {
+    require(lse->is_cuda() && lse->scalar_type() == at::kFloat && lse->is_contiguous() && lse->numel() == b * h,
+            "softmax_lse must be a contiguous CUDA float32 tensor with batch_size * n_heads elements");
+    a.lse_out = lse->data_ptr<float>();
+  }
+  size_t need = 0;
+  check(pat_paged_decode_baseline_workspace_bytes(&a, &need));
+  DeviceScope scope(q);
+  at::Tensor ws = at::empty({(int64_t)need}, at::TensorOptions().dtype(at::kByte).device(q.device()));
+  a.workspace = ws.data_ptr(); a.workspace_bytes = need;
+  check(pat_paged_decode_baseline_launch(&a, raw_stream(q.device())));
+}
+
+}  // namespace
+
+PYBIND11_MODULE(_prefix_attn, m) {
+  m.doc() = "prefix-aware decode attention over a paged KV cache for AMD MI355X (libpat_amd)";
+  require(pat_abi_version() == PAT_ABI_VERSION, "libpat_amd.so and the _prefix_attn extension were built from different headers");
+
+  py::class_<KernelInfo, std::shared_ptr<KernelInfo>>(m, "KernelInfo")
+      .def(py::init<>())
+      .def("to_gpu", [](KernelInfo& ki, const py::object& device) { ki.to_gpu(to_device(device)); }, py::arg("device"))
+      .def_readonly("q_tables", &KernelInfo::q_tables)
+      .def_readonly("block_tables", &KernelInfo::block_tables)
+      .def_readonly("num_seqs_per_CTAs", &KernelInfo::num_seqs)
+      .def_readonly("CTA_ranks", &KernelInfo::ranks)
+      .def_readonly("kv_in_CTAs", &KernelInfo::kvs)
+      // not in the reference: per (box, sequence) the box's ordinal among that sequence's boxes, the
+      // collision-free partial-result slot; and the boxes of this plan per sequence
+      .def_readonly("slot_tables", &KernelInfo::slot_tables)
+      .def_readonly("num_boxes_per_seq", &KernelInfo::num_boxes_per_seq)
+      .def_readonly("max_boxes_per_seq", &KernelInfo::max_boxes)
+      .def_readonly("MNWs", &KernelInfo::mnws)
+      .def_readonly("num_split_per_seq", &KernelInfo::num_split_per_seq)
+      .def_readonly("max_split_per_seq", &KernelInfo::max_split)
+      .def_readonly("max_seqs_in_CTA", &KernelInfo::max_seqs)
+      .def_readonly("max_blocks_in_CTA", &KernelInfo::max_blocks)
+      .def("launch_tables", &KernelInfo::launch_tables,
+           "The per-bucket tables as the kernels get them (boxes longest first, a bucket with a wide head split "
+           "in two) with their tile labels under \"MNWs\" and hints under \"flags\".")
+      .def("launch_position", &KernelInfo::launch_position, py::arg("bucket"),
+           "For the boxes of a scheduler bucket, in scheduler order: (launch bucket, row in it) as two int64 tensors.")
+      .def_property_readonly("_flat", [](const KernelInfo& ki) -> py::object {
+        return ki.flat.has_value() ? py::cast(*ki.flat) : py::none();
+      })
+      .def_property_readonly("_launch_order", [](const KernelInfo& ki) { return ki.launch_order; })
+      .def_property_readonly("_launch_parts", [](const KernelInfo& ki) {
+        std::vector<std::vector<std::tuple<int, int, int>>> out;
+        for (const auto& parts : ki.launch_parts) {
+          out.emplace_back();
+          for (const LaunchPart& p : parts) out.back().emplace_back(p.bucket, p.lo, p.hi);
+        }
+        return out;
+      })
+      .def_property_readonly("_launch_workspace_bytes", [](const KernelInfo& ki) {
+        std::vector<size_t> out;
+        for (const auto& kv : ki.cache) out.push_back(kv.second->need);
+        return out;
+      });
+
+  py::class_<PrefixTreeCPP>(m, "PrefixTreeCPP", py::dynamic_attr())
+      .def(py::init<int>(), py::arg("block_size"))
+      .def_readonly("block_size", &PrefixTreeCPP::block_size)
+      .def("build_radix_tree", &PrefixTreeCPP::build_radix_tree, py::arg("seq_lens"), py::arg("block_table"))
+      .def("pack_schedule", &PrefixTreeCPP::pack_schedule, py::arg("MNWs") = py::none(), py::arg("HRatio") = 1,
+           py::arg("kvHead") = 8, py::arg("use_compute_model") = false)
+      .def_property_readonly("kernel_info", [](const PrefixTreeCPP& t) { return t.info; });
+
+  m.def("prefix_attn_with_kvcache", &fwd_tables, py::arg("q"), py::arg("k_cache_paged"), py::arg("v_cache_paged"),
+        py::arg("num_split_per_seq"), py::arg("query_tables"), py::arg("block_tables"), py::arg("num_seqs_per_CTAs"),
+        py::arg("CTA_ranks"), py::arg("kv_in_CTAs"), py::arg("MNW"), py::arg("max_split_per_seq"),
+        py::arg("max_seqs_in_CTA"), py::arg("max_blocks_in_CTA"), py::arg("softmax_scale"), py::arg("out"),
+        py::arg("timing_") = py::none(), py::kw_only(), py::arg("softmax_lse") = py::none(),
+        py::arg("slot_tables") = py::none(), py::arg("bucket_flags") = py::none(),
+        "Table form. Extra keywords: softmax_lse (float32 [batch, heads]) receives the natural-log LSE; "
+        "slot_tables (KernelInfo.slot_tables) files partial results by each box's ordinal within its sequence "
+        "(derived on the device when absent); bucket_flags are launch-geometry hints.");
+  m.def("prefix_attn_with_kvcache", &fwd_tree, py::arg("q"), py::arg("k_cache_paged"), py::arg("v_cache_paged"),
+        py::arg("tree"), py::arg("softmax_scale"), py::arg("out"), py::kw_only(), py::arg("softmax_lse") = py::none(),
+        "Tree form: the plan of a PrefixTreeCPP whose kernel_info is on the device.");
+  m.def("paged_decode_baseline", &paged_decode_baseline, py::arg("q"), py::arg("k_cache_paged"),
+        py::arg("v_cache_paged"), py::arg("block_table"), py::arg("seq_lens"), py::arg("softmax_scale"), py::arg("out"),
+        py::arg("softmax_lse") = py::none(), py::arg("even_lengths") = false,
+        "Prefix-oblivious paged decode attention through the same kernels: one work item per request.");
+}

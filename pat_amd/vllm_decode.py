@@ -133,7 +133,7 @@ class DecodePlan:
         targets = [(info.kv_in_CTAs, info.block_tables, lambda b, boxes: {b: (boxes, np.arange(len(boxes)))})]
         if launch["kv_in_CTAs"] is not info.kv_in_CTAs:
             if self._launch_row is None:
-                self._launch_row = [info.launch_position(b) for b in range(len(info.MNWs))]
+                self._launch_row = [tuple(t.numpy() for t in info.launch_position(b)) for b in range(len(info.MNWs))]
 
             def in_launch(b, boxes):
                 lb, lr = self._launch_row[b]

@@ -78,3 +78,79 @@ def test_python_plan_sort_for_launch_permutes_rows_only():
         raise AssertionError("expected the tensor form to be refused")
     except ValueError as e:
         assert "before to_tensor" in str(e)
+
+
+def test_extension_is_compiled_and_keeps_the_reference_signatures():
+    # the reference's module is a compiled torch extension (csrc/bindings.cpp:74-158); so is this one
+    from pat_amd import _prefix_attn as ext
+    assert ext.__file__.endswith(".so")
+    assert prefix_attn._prefix_attn is ext
+    import re
+    doc = " ".join(ext.prefix_attn_with_kvcache.__doc__.split())
+    one, two = re.findall(r"\d\. prefix_attn_with_kvcache\((.*?)\) -> None", doc)
+    names = lambda sig: re.findall(r"(?:^|, )(\*|\w+)(?=:|,)", sig)
+    # argument names and order of csrc/bindings.cpp:76-95 and :148-157; keyword-only extras after "*"
+    assert names(one) == ["q", "k_cache_paged", "v_cache_paged", "num_split_per_seq", "query_tables", "block_tables",
+                          "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "MNW", "max_split_per_seq",
+                          "max_seqs_in_CTA", "max_blocks_in_CTA", "softmax_scale", "out", "timing_", "*",
+                          "softmax_lse", "slot_tables", "bucket_flags"]
+    assert "timing_: object = None" in one
+    assert names(two) == ["q", "k_cache_paged", "v_cache_paged", "tree", "softmax_scale", "out", "*", "softmax_lse"]
+    t = ext.PrefixTreeCPP(block_size=16)
+    assert t.block_size == 16 and t.kernel_info.MNWs == []
+    sig = " ".join(ext.PrefixTreeCPP.pack_schedule.__doc__.split())
+    assert re.search(r"MNWs: object = None, HRatio: [\w.]+ = 1, kvHead: [\w.]+ = 8, use_compute_model: bool = False", sig), sig
+
+
+def test_extension_maps_planner_errors_to_python_exceptions():
+    import pytest
+    from pat_amd import PrefixTreeCPP
+    t = PrefixTreeCPP(16)
+    t.build_radix_tree([64, 64], torch.tensor([[0, 1, 2, 3], [0, 1, 4, 5]], dtype=torch.int32))
+    with pytest.raises(KeyError):
+        t.pack_schedule([[64, 128, 4], [16, 128, 1]], 1, 8)      # computed bucket not offered
+    with pytest.raises(ZeroDivisionError):
+        t.pack_schedule(None, 0, 8)
+    empty = PrefixTreeCPP(16)
+    empty.build_radix_tree([], torch.zeros(0, 1, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        empty.pack_schedule(None, 1, 8)                          # max() of an empty batch
+    t.pack_schedule([], 1, 8)                                     # an empty list selects the default buckets
+    assert t.kernel_info.max_split_per_seq >= 1
+    with pytest.raises(TypeError):
+        prefix_attn.prefix_attn_with_kvcache(torch.zeros(1), torch.zeros(1), torch.zeros(1), "not a tree", 1.0,
+                                             torch.zeros(1))
+
+
+def test_planner_calls_release_the_gil():
+    # build_radix_tree / pack_schedule run without the GIL (csrc/bindings.cpp:124,138): a Python
+    # thread makes progress while another one plans a large batch
+    import threading
+    import time
+    from pat_amd import PrefixTreeCPP
+    n, width = 4096, 512
+    table = torch.arange(n * width, dtype=torch.int32).view(n, width)
+    table[:, :256] = torch.arange(256, dtype=torch.int32)          # a shared prefix
+    lens = [width * 16] * n
+    ticks, stop = [0], threading.Event()
+
+    def spin():
+        while not stop.is_set():
+            ticks[0] += 1
+            time.sleep(0)
+
+    th = threading.Thread(target=spin)
+    th.start()
+    try:
+        time.sleep(0.02)
+        before, t0 = ticks[0], time.perf_counter()
+        tree = PrefixTreeCPP(16)
+        tree.build_radix_tree(lens, table)
+        tree.pack_schedule(None, 4, 8)
+        native_s, during = time.perf_counter() - t0, ticks[0] - before
+    finally:
+        stop.set()
+        th.join()
+    assert tree.kernel_info.num_split_per_seq.numel() == n
+    # with the GIL held throughout, the other thread would get at most a few switches
+    assert during > 20 or native_s < 0.005, (during, native_s)

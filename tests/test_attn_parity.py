@@ -175,7 +175,7 @@ def test_merge_of_more_than_256_slots(tuning):
     # merge kernel's loops past its 256 register-held slots run
     print("[case] merge of 320 slots per row", flush=True)
     import ctypes as C
-    from pat_amd import _lib, _prefix_attn
+    from pat_amd import _ctypes_launch, _lib
     dev = _device()
     nxt = [0]
 
@@ -205,13 +205,13 @@ def test_merge_of_more_than_256_slots(tuning):
     tuning(chunk_tokens=32, tall_chunk_tokens=32)
     out = torch.full_like(q, float("nan"))
     lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
-    L = _prefix_attn._prepare(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+    L = _ctypes_launch.prepare(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
                               ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
                               ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, lse)
     geo = _lib.FwdGeometry()
     assert _lib.load().pat_fwd_geometry_of(C.byref(L.args), C.byref(geo)) == 0
     assert geo.num_slots == 5 * 64
-    _prefix_attn._run(L, dev)
+    _ctypes_launch.run(L, dev)
     torch.cuda.synchronize()
     ref_out, ref_lse = _oracle(w, q, k, v)
     _assert_close("320 slots", out, lse, ref_out, ref_lse, w.dtype)
@@ -248,7 +248,7 @@ def test_single_slot_launch_writes_out_directly(case, tuning):
     # (csrc/api.h:230-238 does the same for max_split_per_seq == 1). All three epilogues. (Batches
     # of 27 boxes or more: below that the balancer halves boxes and every row has two slots.)
     print(f"[case] direct output, {case}", flush=True)
-    from pat_amd import _prefix_attn
+    from pat_amd import _ctypes_launch
     dev = _device()
     if case == "combine":          # few boxes of a few steps: 4 waves share a box, states combined in LDS
         w = workloads.independent("direct-a", 32, 300, 32, 8, 128, torch.bfloat16, 5)
@@ -271,12 +271,12 @@ def test_single_slot_launch_writes_out_directly(case, tuning):
         tuning(direct_out=1 if direct else 0)
         out = torch.full_like(q, float("nan"))
         lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
-        L = _prefix_attn._prepare(q, k, v, info.num_split_per_seq, lt["q_tables"], lt["block_tables"],
+        L = _ctypes_launch.prepare(q, k, v, info.num_split_per_seq, lt["q_tables"], lt["block_tables"],
                                   lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
                                   info.max_split_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
                                   1.0 / math.sqrt(w.head_dim), out, lse, lt.get("slot_tables"), lt.get("flags"))
         assert (L.need == 0) == direct, f"direct {direct}: workspace {L.need} bytes"
-        _prefix_attn._run(L, dev)
+        _ctypes_launch.run(L, dev)
         torch.cuda.synchronize()
         return out, lse
 
@@ -293,7 +293,7 @@ def test_single_slot_launch_with_strided_out(pad):
     # `out` as a view with padded head rows: 8 extra elements keep 8-byte stores possible (direct
     # route), 2 do not (the launch falls back to partial slots + merge); same result either way
     print(f"[case] direct output into a strided view, head rows padded by {pad}", flush=True)
-    from pat_amd import _prefix_attn
+    from pat_amd import _ctypes_launch
     dev = _device()
     w = workloads.independent("direct-s", 48, 400, 32, 8, 128, torch.float16, 9)
     q, k, v = w.tensors(dev)
@@ -306,9 +306,7 @@ def test_single_slot_launch_with_strided_out(pad):
     lse = torch.empty(w.batch, w.heads, dtype=torch.float32, device=dev)
     prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
     torch.cuda.synchronize()
-    info = tree.kernel_info
-    L = next(iter(info._launch_cache.values()))
-    assert (L.need == 0) == (pad == 8)
+    assert (tree.kernel_info._launch_workspace_bytes == [0]) == (pad == 8)
     assert torch.isnan(big[..., w.head_dim:]).all(), "the padding of the view must stay untouched"
     ref_out, ref_lse = _oracle(w, q, k, v)
     _assert_close(f"direct/strided{pad}", out, lse, ref_out, ref_lse, w.dtype)

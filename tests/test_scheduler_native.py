@@ -144,34 +144,75 @@ def test_error_mapping():
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5a"])
 def test_flat_plan_equals_the_per_table_view(name):
     """The one-buffer form of the plan (pat_tree_flat_plan: scheduler-order tables + launch copies,
-    sorted and split by the planner) against the per-table view with the launch copies built in
-    Python: same tables, same launch order, same parts."""
+    sorted and split by the planner) against the ragged plan of the Python-level `PrefixTree` and a
+    launch order derived here: same tables, same order, same parts."""
+    import numpy as np
     from pat_amd import PrefixTreeCPP, workloads
-    from pat_amd._prefix_attn import KernelInfo
     w = workloads.make(name, seed=1)
     t = PrefixTreeCPP(w.page_size)
     t.build_radix_tree(w.seq_lens, w.padded_table())
     t.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
     flat = t.kernel_info
     assert flat._flat is not None and flat._flat.dim() == 1
-    view = KernelInfo._from_view(t._native.plan_view())
-    assert flat.MNWs == view.MNWs and flat.max_split_per_seq == view.max_split_per_seq
-    assert flat.max_seqs_in_CTA == view.max_seqs_in_CTA and flat.max_blocks_in_CTA == view.max_blocks_in_CTA
-    assert torch.equal(flat.num_split_per_seq, view.num_split_per_seq)
-    names = ("q_tables", "block_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "slot_tables")
-    for key in names:
-        assert all(torch.equal(a, b) for a, b in zip(getattr(flat, key), getattr(view, key))), key
-    fl, vl = flat.launch_tables(), view.launch_tables()
-    assert fl["MNWs"] == vl["MNWs"]
-    for key in names:
-        assert len(fl[key]) == len(vl[key]) and all(torch.equal(a, b) for a, b in zip(fl[key], vl[key])), key
-    assert flat._launch_parts == view._launch_parts
-    assert all(torch.equal(a.long(), b) for a, b in zip(flat._launch_order, view._launch_order))
+    p = PrefixTree(w.page_size)
+    p.build_radix_tree(w.seq_lens, w.rows)
+    ref = p.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    assert flat.MNWs == ref.MNWs and flat.max_split_per_seq == ref.max_split_per_seq
+    assert flat.max_seqs_in_CTA == ref.max_seqs_in_CTA and flat.max_blocks_in_CTA == ref.max_blocks_in_CTA
+    assert flat.num_split_per_seq.tolist() == ref.num_split_per_seq
+    assert flat.num_boxes_per_seq.tolist() == ref.num_split_per_seq     # first pack: the counts agree
+    assert flat.max_boxes_per_seq == ref.max_split_per_seq
+
+    def padded(rows, width):
+        return [list(r) + [0] * (width - len(r)) for r in rows]
+
+    for b in range(len(ref.MNWs)):
+        assert flat.q_tables[b].tolist() == padded(ref.q_tables[b], flat.q_tables[b].shape[1])
+        assert flat.slot_tables[b].tolist() == padded(ref.slot_tables[b], flat.q_tables[b].shape[1])
+        assert flat.block_tables[b].tolist() == padded(ref.block_tables[b], flat.block_tables[b].shape[1])
+        assert flat.num_seqs_per_CTAs[b].tolist() == ref.num_seqs_per_CTAs[b]
+        assert flat.CTA_ranks[b].tolist() == ref.CTA_ranks[b]
+        assert flat.kv_in_CTAs[b].tolist() == ref.kv_in_CTAs[b]
+    # launch copies: boxes longest first (stable); a bucket whose wide head (at most a quarter of the
+    # boxes, each more than twice as long as any other) is split off, the rest with a narrower table
+    launch = flat.launch_tables()
+    parts = flat._launch_parts
+    at = 0
+    for b in range(len(ref.MNWs)):
+        kv = np.asarray(ref.kv_in_CTAs[b])
+        order = np.argsort(-kv, kind="stable")
+        assert flat._launch_order[b].tolist() == order.tolist()
+        n = len(kv)
+        k = int((kv[order] > kv[order][0] // 2).sum())
+        cuts = [0, k, n] if (n >= 4 and 0 < k <= n // 4) else [0, n]
+        assert [(lo, hi) for _, lo, hi in parts[b]] == list(zip(cuts[:-1], cuts[1:]))
+        for lb, lo, hi in parts[b]:
+            assert lb == at
+            at += 1
+            rows = torch.as_tensor(order[lo:hi].copy())
+            assert launch["MNWs"][lb] == ref.MNWs[b]
+            lw = launch["block_tables"][lb].shape[1]
+            if lo > 0:
+                longest = max(len(ref.block_tables[b][i]) for i in order[lo:hi])
+                assert lw == min(flat.block_tables[b].shape[1], longest + 8)
+            else:
+                assert lw == flat.block_tables[b].shape[1]
+            assert torch.equal(launch["block_tables"][lb], flat.block_tables[b][rows][:, :lw])
+            for key, src in (("q_tables", flat.q_tables), ("slot_tables", flat.slot_tables),
+                             ("num_seqs_per_CTAs", flat.num_seqs_per_CTAs), ("CTA_ranks", flat.CTA_ranks),
+                             ("kv_in_CTAs", flat.kv_in_CTAs)):
+                assert torch.equal(launch[key][lb], src[b][rows]), key
+        pos_b, pos_r = flat.launch_position(b)
+        for lb, lo, hi in parts[b]:
+            assert pos_b[order[lo:hi]].tolist() == [lb] * (hi - lo)
+            assert pos_r[order[lo:hi]].tolist() == list(range(hi - lo))
+    assert at == len(launch["MNWs"])
     if name == "c4":
-        assert max(len(p) for p in flat._launch_parts) == 2      # a bucket with a wide head
+        assert max(len(p) for p in parts) == 2      # a bucket with a wide head
     # the device copy is one buffer too and its views line up
+    before = [x.clone() for x in launch["kv_in_CTAs"]]
     flat.to_gpu("cpu")
-    assert torch.equal(flat.launch_tables()["kv_in_CTAs"][0], vl["kv_in_CTAs"][0])
+    assert all(torch.equal(a, b) for a, b in zip(flat.launch_tables()["kv_in_CTAs"], before))
 
 
 def test_flat_plan_marks_even_buckets():

@@ -8,7 +8,7 @@ import math
 import pytest
 import torch
 
-from pat_amd import PrefixTreeCPP, _lib, _prefix_attn, workloads
+from pat_amd import PrefixTreeCPP, _ctypes_launch, _lib, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -26,7 +26,7 @@ def _both_routes(name, w, dev):
     for static in (False, True):
         out = torch.full_like(q, float("nan"))
         lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
-        L = _prefix_attn._prepare(q, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
+        L = _ctypes_launch.prepare(q, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
                                   lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
                                   info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
                                   1.0 / math.sqrt(w.head_dim), out, lse, lt["slot_tables"], lt.get("flags"))
