@@ -13,7 +13,10 @@ Prints ONE JSON line. `value` is unique-KV bytes / time per call (GB/s); `ms_per
 latency per call. `roofline` covers the split kernel (HBM-bound): algorithmic bytes = unique
 KV bytes of the batch, duration = mean split-kernel time from HIP events on the launch stream.
 `cpu_baseline` times this repository's CPU restatement of the reference's PyTorch attention
-on the host cores.
+on the host cores. `api_us_per_call` is the same loop through the drop-in call
+`prefix_attn_with_kvcache(q, k, v, tree, scale, out)` of the compiled extension (workspace from
+torch's allocator per call). The default run (workload c2) also measures the other five benchmark
+workloads, more briefly, and lists them under `configs`.
 """
 from __future__ import annotations
 
@@ -30,9 +33,26 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 INFINITY_CACHE_BYTES = 256 << 20
-# HBM bytes per split-kernel launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by
-# the same counter's reading for a 1 GiB copy kernel (profiles/pat_split_kernel_<workload>.md)
-MEASURED_TRAFFIC_BYTES = {"c2": 95_800_000, "c5b": 541_800_000}
+
+
+def measured_traffic_bytes(workload: str, seed: int):
+    """HBM bytes per split-kernel launch as rocprofv3 measured them (--pmc FETCH_SIZE + WRITE_SIZE, each
+    scaled by the same counter's reading for a 1 GiB copy kernel), from the marker line of
+    profiles/pat_split_kernel_<workload>.md. None when there is no such measurement for this
+    workload and seed, or when the kernel sources have changed since it was taken."""
+    import hashlib
+    import re
+    path = os.path.join(ROOT, "profiles", f"pat_split_kernel_{workload}.md")
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"bench-marker: workload=(\S+) seed=(\d+) traffic_bytes=(\d+) kernel_sources_sha256=([0-9a-f]+)",
+                  open(path).read())
+    if m is None or m.group(1) != workload or int(m.group(2)) != seed:
+        return None
+    h = hashlib.sha256()
+    for rel in ("pat_amd/csrc/hip/pat_split.hip", "pat_amd/csrc/hip/fwd_params.hpp", "pat_amd/csrc/capi_fwd.hip"):
+        h.update(open(os.path.join(ROOT, rel), "rb").read())
+    return int(m.group(3)) if h.hexdigest() == m.group(4) else None
 
 WORKLOAD_TEXT = {
     "c1": "8 req, 256 shared + 32 private tokens, 8/8 heads, d64, fp16",
@@ -71,46 +91,16 @@ class Hip:
         return out.value
 
 
-def main() -> None:
-    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOAD_TEXT))
-    ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-oblivious", action="store_true")
-    ap.add_argument("--kernel-loop-only", action="store_true",
-                    help="run only warmup + timed steps (for rocprofv3 runs)")
-    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
-                    help="instead of the benchmark, run a plain elementwise copy of this many MiB 5 times "
-                         "(reads N, writes N bytes): the known-size kernel that scales rocprofv3's "
-                         "FETCH_SIZE / WRITE_SIZE readings")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (the path has no cross-GPU step); use --gpus 1",
-              file=sys.stderr)
-        sys.exit(2)
-
+def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
+    """One workload: plan, timed C-ABI loop, per-kernel event times, the drop-in API loop, the
+    prefix-oblivious comparator and (headline only) the CPU baseline."""
     import torch
-    from pat_amd import PrefixTreeCPP, _ctypes_launch, _lib, workloads
+    from pat_amd import PrefixTreeCPP, _ctypes_launch, _lib, prefix_attn_with_kvcache, workloads
 
-    assert torch.cuda.is_available(), "bench.py needs an AMD GPU"
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if a.calibrate_copy_mib > 0:
-        n = a.calibrate_copy_mib << 20
-        src = torch.ones(n // 4, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            torch.mul(src, 1.0, out=dst)        # one elementwise kernel: reads n bytes, writes n bytes
-        torch.cuda.synchronize()
-        print(json.dumps({"calibration_copy_bytes": n, "launches": 5}))
-        return
     lib = _lib.load()
     hip = Hip()
-
-    w = workloads.make(a.workload, seed=a.seed)
+    w = workloads.make(workload, seed=a.seed)
     cache_bytes = w.kv_bytes(w.num_blocks * w.page_size)
     copies = max(2, min(16, math.ceil(2.5 * INFINITY_CACHE_BYTES / cache_bytes)))
     q, ks, vs = w.tensors(dev, copies=copies)
@@ -173,13 +163,12 @@ def main() -> None:
         torch.cuda.synchronize()
         return (time.perf_counter() - t) * 1e3 / steps
 
-    ms_per_step = timed(pat_launches, a.steps, a.warmup)
+    ms_per_step = timed(pat_launches, steps, warmup)
     if a.kernel_loop_only:
-        print(json.dumps({"ms_per_step": ms_per_step, "steps": a.steps, "warmup": a.warmup}))
-        return
+        return {"ms_per_step": ms_per_step, "steps": steps, "warmup": warmup}
 
     # per-kernel durations from HIP events on the launch stream (same step sequence)
-    n_ev = min(a.steps, 100)
+    n_ev = min(steps, 100)
     ev = [(hip.event(), hip.event(), hip.event()) for _ in range(n_ev)]
     for i, (e0, e1, e2) in enumerate(ev):
         L = pat_launches[i % copies]
@@ -213,15 +202,15 @@ def main() -> None:
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f16",
         "data": "synthetic",
-        "config": {"workload": f"{a.workload}: {WORKLOAD_TEXT[a.workload]}", "batch": w.batch,
+        "config": {"workload": f"{workload}: {WORKLOAD_TEXT[workload]}", "batch": w.batch,
                    "heads": w.heads, "kv_heads": w.kv_heads, "head_dim": w.head_dim, "page_size": w.page_size,
                    "seed": a.seed, "unique_kv_tokens": w.unique_tokens, "total_kv_tokens": w.total_tokens,
                    "kv_cache_copies_rotated": copies, "tree": w.tree},
@@ -244,18 +233,32 @@ def main() -> None:
                      "traffic": None},
     }
 
-    if a.seed == 0:
-        result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.workload)
+    result["roofline"]["traffic"] = measured_traffic_bytes(workload, a.seed)
+
+    # the same steps through the drop-in call of the compiled extension (tree form): argument checks
+    # and launch preparation are cached per (q, k, v, out), the workspace comes from torch's
+    # caching allocator at every call
+    def api_step(i):
+        prefix_attn_with_kvcache(q, ks[i % copies], vs[i % copies], tree, scale, out)
+
+    for i in range(max(warmup, copies)):
+        api_step(i)
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for i in range(steps):
+        api_step(i)
+    torch.cuda.synchronize()
+    result["api_us_per_call"] = round((time.perf_counter() - t) * 1e6 / steps, 3)
 
     if not a.no_oblivious:
         ob = workloads.oblivious_plan(w, dev)
         ob_kw = {k: ob[k] for k in pat_kw}
         ob_launches, ob_ws = prepare(ob_kw, None)
-        ob_ms = timed(ob_launches, a.steps, a.warmup)
+        ob_ms = timed(ob_launches, steps, warmup)
         result["oblivious_us_per_call"] = round(ob_ms * 1e3, 3)
         result["speedup_vs_oblivious"] = round(ob_ms / ms_per_step, 3)
 
-    if not a.no_cpu_baseline:
+    if headline and not a.no_cpu_baseline:
         from oracle import attn_oracle
         qc, kc, vc = q.cpu(), ks[0].cpu(), vs[0].cpu()
         cores = os.cpu_count() or 1
@@ -272,8 +275,63 @@ def main() -> None:
         result["cpu_baseline"] = {"value": round(unique_bytes / cpu_s / 1e9, 4), "unit": "GB/s",
                                   "cores": torch.get_num_threads(), "kind": "port",
                                   "us_per_call": round(cpu_s * 1e6, 1),
-                                  "sample": f"whole {a.workload} batch, fp32 PyTorch restatement of the reference's "
+                                  "sample": f"whole {workload} batch, fp32 PyTorch restatement of the reference's "
                                             f"attention_ref over gathered dense KV, mean of {runs} runs after 1 warm-up"}
+    return result
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOAD_TEXT))
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-oblivious", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="do not measure the other benchmark workloads beside the named one")
+    ap.add_argument("--kernel-loop-only", action="store_true",
+                    help="run only warmup + timed steps (for rocprofv3 runs)")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="instead of the benchmark, run a plain elementwise copy of this many MiB 5 times "
+                         "(reads N, writes N bytes): the known-size kernel that scales rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no cross-GPU step); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs an AMD GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if a.calibrate_copy_mib > 0:
+        n = a.calibrate_copy_mib << 20
+        src = torch.ones(n // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)        # one elementwise kernel: reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_copy_bytes": n, "launches": 5}))
+        return
+    steps, warmup = a.steps, a.warmup
+    result = measure(a, a.workload, steps, warmup, headline=True)
+    if a.workload == "c2" and not a.no_configs and not a.kernel_loop_only:
+        # the other benchmark workloads, measured the same way (fewer steps; CPU baseline for c2 only)
+        result["configs"] = []
+        for name in ("c1", "c3", "c4", "c5a", "c5b"):
+            r = measure(a, name, max(20, min(steps, 100)), warmup, headline=False)
+            result["configs"].append({
+                "workload": r["config"]["workload"], "us_per_call": r["us_per_call"],
+                "api_us_per_call": r["api_us_per_call"], "unique_kv_gbps": r["value"],
+                "pct_of_hbm_peak": r["pct_of_hbm_peak"], "split_us": r["event_us"]["split_mean"],
+                "merge_us": r["event_us"]["merge_mean"], "frac": r["roofline"]["frac"],
+                "oblivious_us_per_call": r.get("oblivious_us_per_call"),
+                "speedup_vs_oblivious": r.get("speedup_vs_oblivious"), "workgroups": r["geometry"]["workgroups"],
+                "dtype": r["dtype"]})
     print(json.dumps(result))
 
 
