@@ -117,16 +117,19 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     out = torch.empty_like(q)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
-    def prepare(plan_kw, slots):
-        launches = []
+    def prepare(plan_kw, slots, autotune):
+        # One measured geometry per plan (pat_fwd_autotune, what the drop-in call does the first time
+        # it sees a plan shape), shared by the launches over the rotated cache copies.
+        launches, tuning = [], None
         for i in range(copies):
             L = _ctypes_launch.prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
-                                      plan_kw["block_tables"], plan_kw["num_seqs_per_CTAs"], plan_kw["CTA_ranks"],
-                                      plan_kw["kv_in_CTAs"], plan_kw["MNW"], plan_kw["max_split_per_seq"],
-                                      plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots,
-                                      plan_kw.get("bucket_flags"))
+                                       plan_kw["block_tables"], plan_kw["num_seqs_per_CTAs"], plan_kw["CTA_ranks"],
+                                       plan_kw["kv_in_CTAs"], plan_kw["MNW"], plan_kw["max_split_per_seq"],
+                                       plan_kw["max_seqs_in_CTA"], plan_kw["max_blocks_in_CTA"], scale, out, None, slots,
+                                       plan_kw.get("bucket_flags"), autotune=autotune and i == 0, tuning=tuning)
+            tuning = L.tuning
             launches.append(L)
-        ws = torch.empty(max(L.need for L in launches), dtype=torch.uint8, device=dev)
+        ws = torch.empty(max(max(L.need for L in launches), 256), dtype=torch.uint8, device=dev)
         for L in launches:
             L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), ws.numel()
         return launches, ws
@@ -137,7 +140,7 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
                   CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=lt["MNWs"],
                   max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                   max_blocks_in_CTA=info.max_blocks_in_CTA, bucket_flags=lt.get("flags"))
-    pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"])
+    pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"], not a.no_autotune)
 
     def step(launches, i):
         rc = lib.pat_fwd_launch(C.byref(launches[i % copies].args), C.c_void_p(stream))
@@ -228,6 +231,12 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
         "geometry": {"chunk_tokens": geo.chunk_tokens, "tall_chunk_tokens": geo.tall_chunk_tokens,
                      "chunks_per_rank": geo.chunks_per_rank, "workgroups": geo.num_workgroups},
         "plan_build_ms_host": round(plan_ms, 3),
+        # the measured choice of the launch geometry (made once per plan shape, outside the timed
+        # region, like the plan itself): overrides in pat_fwd_tuning's field order, null = none
+        "autotune": None if a.no_autotune else {
+            "chosen": (None if pat_launches[0].tuning is None else
+                       {f: getattr(pat_launches[0].tuning, f) for f, _ in _lib.FwdTuning._fields_}),
+            "tuning_run_us": {"chosen": round(pat_launches[0].tuned_us, 2), "automatic": round(pat_launches[0].auto_us, 2)}},
         "roofline": {"bound": "hbm", "kernel": "pat_split_kernel", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": None},
@@ -253,7 +262,7 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     if not a.no_oblivious:
         ob = workloads.oblivious_plan(w, dev)
         ob_kw = {k: ob[k] for k in pat_kw}
-        ob_launches, ob_ws = prepare(ob_kw, None)
+        ob_launches, ob_ws = prepare(ob_kw, None, not a.no_autotune)
         ob_ms = timed(ob_launches, steps, warmup)
         result["oblivious_us_per_call"] = round(ob_ms * 1e3, 3)
         result["speedup_vs_oblivious"] = round(ob_ms / ms_per_step, 3)
@@ -289,6 +298,8 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-oblivious", action="store_true")
+    ap.add_argument("--no-autotune", action="store_true",
+                    help="launch geometry from sizes alone, without the measured choice the drop-in call makes")
     ap.add_argument("--no-configs", action="store_true",
                     help="do not measure the other benchmark workloads beside the named one")
     ap.add_argument("--kernel-loop-only", action="store_true",

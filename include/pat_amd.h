@@ -238,6 +238,26 @@ typedef struct pat_fwd_bucket {
  * A wrong hint costs time, never correctness. */
 #define PAT_BUCKET_EVEN 1
 
+/* Overrides of the launch geometry. pat_fwd_set_tuning sets them process-wide (a tuning and test
+ * aid, not meant to change while launches are in flight on other threads); pat_fwd_args.tuning sets
+ * them for one launch (what pat_fwd_autotune's result is for). 0 / -1 = automatic, as noted per field. The
+ * initial values come from the environment variables PAT_CHUNK_TOKENS, PAT_TALL_CHUNK_TOKENS,
+ * PAT_HEAD_PER_WAVE_TOKENS, PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS,
+ * PAT_EQUALIZE_CHUNKS, PAT_DIRECT_OUT, read once; pat_fwd_set_tuning(NULL) reads them again. */
+typedef struct pat_fwd_tuning {
+  int32_t chunk_tokens;              /* KV tokens per workgroup, boxes <= 16 rows (0: automatic)   */
+  int32_t tall_chunk_tokens;         /* same for boxes of 17..64 rows (0: automatic)                */
+  int32_t head_per_wave_tokens;      /* widest box of a bucket that runs a kv head per wave         */
+                                     /* (-1: automatic, 0: never)                                   */
+  int32_t head_per_wave_long_tokens; /* chunk of long boxes run a kv head per wave (0: automatic)   */
+  int64_t head_per_wave_long_wgs;    /* such workgroups a bucket needs for that (-1: automatic)     */
+  int32_t equalize_chunks;           /* even chunks per box: -1 automatic, 0 never, 1 always        */
+  int32_t direct_out;                /* single-slot launches write `out` from the split kernel:     */
+                                     /* -1 / 1 when possible, 0 never                               */
+} pat_fwd_tuning;
+int pat_fwd_set_tuning(const pat_fwd_tuning* tuning);
+int pat_fwd_get_tuning(pat_fwd_tuning* out);
+
 /* Mirrors the arguments of pat_mha_fwd_kvcache (csrc/api.h:110-127).
  * Strides are in ELEMENTS (as csrc/api.h:43); the last dimension of q, k, v, out
  * must be contiguous. Unlike the reference, V may have strides of its own.
@@ -272,6 +292,8 @@ typedef struct pat_fwd_args {
   size_t workspace_bytes;
   void* split_done_event;        /* optional hipEvent_t recorded on the stream between the   */
                                  /* split kernel and the merge kernel (timing aid), or NULL  */
+  const pat_fwd_tuning* tuning;  /* optional launch-geometry overrides for this call (host    */
+                                 /* memory, read during the call); NULL: the process-wide ones */
 } pat_fwd_args;
 
 /* Argument checks of csrc/api.h:129-181 that need no GPU (dtype enum, head_dim,
@@ -325,24 +347,25 @@ int pat_fwd_slots_bytes(const pat_fwd_args* args, size_t* bytes);
 int pat_fwd_derive_slots(const pat_fwd_args* args, void* buffer, size_t buffer_bytes,
                          int64_t* bucket_offsets, void* hip_stream);
 
-/* Overrides of the launch geometry: a tuning and test aid, process-wide, not meant to change
- * while launches are in flight on other threads. 0 / -1 = automatic, as noted per field. The
- * initial values come from the environment variables PAT_CHUNK_TOKENS, PAT_TALL_CHUNK_TOKENS,
- * PAT_HEAD_PER_WAVE_TOKENS, PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS,
- * PAT_EQUALIZE_CHUNKS, PAT_DIRECT_OUT, read once; pat_fwd_set_tuning(NULL) reads them again. */
-typedef struct pat_fwd_tuning {
-  int32_t chunk_tokens;              /* KV tokens per workgroup, boxes <= 16 rows (0: automatic)   */
-  int32_t tall_chunk_tokens;         /* same for boxes of 17..64 rows (0: automatic)                */
-  int32_t head_per_wave_tokens;      /* widest box of a bucket that runs a kv head per wave         */
-                                     /* (-1: automatic, 0: never)                                   */
-  int32_t head_per_wave_long_tokens; /* chunk of long boxes run a kv head per wave (0: automatic)   */
-  int64_t head_per_wave_long_wgs;    /* such workgroups a bucket needs for that (-1: automatic)     */
-  int32_t equalize_chunks;           /* even chunks per box: -1 automatic, 0 never, 1 always        */
-  int32_t direct_out;                /* single-slot launches write `out` from the split kernel:     */
-                                     /* -1 / 1 when possible, 0 never                               */
-} pat_fwd_tuning;
-int pat_fwd_set_tuning(const pat_fwd_tuning* tuning);
-int pat_fwd_get_tuning(pat_fwd_tuning* out);
+
+/* Measured choice of the launch geometry (no counterpart in the reference, whose tile shapes are
+ * fixed per bucket). The best chunking of a launch depends on how its workgroups share the CUs,
+ * which sizes alone do not predict for mid-size launches; pat_fwd_autotune runs the launch `reps`
+ * times (after 2 untimed runs) under each of a few candidate geometries - the automatic one first -
+ * on `hip_stream`, times them with HIP events, and stores in *best the overrides of the fastest
+ * (the automatic values unless a candidate beats them by 4 % and 1 us). Pass the result as
+ * pat_fwd_args.tuning of later launches with the same plan shape. `out` holds a valid result
+ * afterwards. args->workspace must hold pat_fwd_autotune_workspace_bytes() bytes (the largest
+ * candidate's need). `evict` (optional): a device buffer at least as large as the memory-side cache
+ * (256 MB on MI355X) that is read before every timed launch, outside its interval, so that each runs
+ * against HBM, as the layers of a model, each with a KV cache of its own, do; with NULL the launches
+ * are timed back to back and inputs that fit the cache look faster than they will be. The call
+ * SYNCHRONISES the stream (not for use under graph capture) and creates and destroys two HIP
+ * events. best_us / auto_us (optional) receive the time per launch of the chosen and of the
+ * automatic geometry. */
+int pat_fwd_autotune_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
+int pat_fwd_autotune(const pat_fwd_args* args, void* hip_stream, int32_t reps, const void* evict,
+                     size_t evict_bytes, pat_fwd_tuning* best, float* best_us, float* auto_us);
 
 /* Description of the launch geometry chosen for `args` (for benchmarks/tests). */
 typedef struct pat_fwd_geometry {

@@ -29,11 +29,11 @@ def _strides3(t: torch.Tensor):
 
 class _Launch:
     """A prepared pat_fwd_args (+ the tensors it points into, kept alive)."""
-    __slots__ = ("args", "buckets", "keep", "workspace", "need")
+    __slots__ = ("args", "buckets", "keep", "workspace", "need", "tuning", "tuned_us", "auto_us")
 
 
 def prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MNW, max_split,
-            max_seqs, max_blocks, scale, out, lse, slot_tables=None, bucket_flags=None) -> _Launch:
+            max_seqs, max_blocks, scale, out, lse, slot_tables=None, bucket_flags=None, autotune=False, tuning=None) -> _Launch:
     lib = _lib.load()
     # --- checks that need tensor metadata (csrc/api.h:131-181, :256-277) -----------------
     _check(q.dtype in (torch.float16, torch.bfloat16), "only support fp16 and bf16 data type")
@@ -116,6 +116,25 @@ def prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MN
         for i in range(nb):
             L.buckets[i].q_slot = derived.data_ptr() + 4 * offsets[i]
         a.num_split_per_seq = derived.data_ptr()
+    L.tuning, L.tuned_us, L.auto_us = tuning, None, None
+    if tuning is not None:          # a geometry measured earlier for this plan shape
+        a.tuning = C.pointer(L.tuning)
+    elif autotune:
+        # measured choice of the launch geometry (pat_fwd_autotune): runs the launch a few times per
+        # candidate on the current stream and synchronises it; `out` holds a valid result afterwards
+        most = C.c_size_t(0)
+        _lib.check(lib.pat_fwd_autotune_workspace_bytes(C.byref(a), C.byref(most)))
+        scratch = torch.empty(max(most.value, 256), dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = scratch.data_ptr(), scratch.numel()
+        L.tuning = _lib.FwdTuning()
+        best_us, auto_us = C.c_float(0), C.c_float(0)
+        evict = _evict_buffer(q.device)
+        _lib.check(lib.pat_fwd_autotune(C.byref(a), C.c_void_p(_raw_stream(q.device.index)), 10,
+                                        C.c_void_p(evict.data_ptr()), evict.numel(), C.byref(L.tuning),
+                                        C.byref(best_us), C.byref(auto_us)))
+        a.tuning = C.pointer(L.tuning)
+        a.workspace, a.workspace_bytes = None, 0
+        L.tuned_us, L.auto_us = best_us.value, auto_us.value
     need = C.c_size_t(0)
     _lib.check(lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)))
     L.args, L.need = a, need.value
@@ -125,6 +144,17 @@ def prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MN
               None if slot_tables is None else list(slot_tables), derived)
     L.workspace = None
     return L
+
+
+_EVICT: dict = {}
+
+
+def _evict_buffer(device: torch.device) -> torch.Tensor:
+    """Per device: 320 MB that the tuning run reads between timed launches (larger than the 256 MB
+    memory-side cache), allocated on first use and kept."""
+    if device.index not in _EVICT:
+        _EVICT[device.index] = torch.zeros(320 << 20, dtype=torch.uint8, device=device)
+    return _EVICT[device.index]
 
 
 def _raw_stream(index: int) -> int:

@@ -96,6 +96,17 @@ class BaselineArgs(C.Structure):
                 ("workspace_bytes", C.c_size_t)]
 
 
+class FwdTuning(C.Structure):
+    _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
+                ("head_per_wave_tokens", C.c_int32), ("head_per_wave_long_tokens", C.c_int32),
+                ("head_per_wave_long_wgs", C.c_int64), ("equalize_chunks", C.c_int32),
+                ("direct_out", C.c_int32)]
+
+    @classmethod
+    def automatic(cls) -> "FwdTuning":
+        return cls(0, 0, -1, 0, -1, -1, -1)
+
+
 class FwdArgs(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("batch", C.c_int32), ("seqlen_q", C.c_int32),
                 ("heads", C.c_int32), ("kv_heads", C.c_int32), ("head_dim", C.c_int32),
@@ -109,18 +120,7 @@ class FwdArgs(C.Structure):
                 ("max_blocks_in_box", C.c_int32), ("softmax_scale", C.c_float),
                 ("num_buckets", C.c_int32), ("buckets", C.POINTER(FwdBucket)),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-                ("split_done_event", C.c_void_p)]
-
-
-class FwdTuning(C.Structure):
-    _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
-                ("head_per_wave_tokens", C.c_int32), ("head_per_wave_long_tokens", C.c_int32),
-                ("head_per_wave_long_wgs", C.c_int64), ("equalize_chunks", C.c_int32),
-                ("direct_out", C.c_int32)]
-
-    @classmethod
-    def automatic(cls) -> "FwdTuning":
-        return cls(0, 0, -1, 0, -1, -1, -1)
+                ("split_done_event", C.c_void_p), ("tuning", C.POINTER(FwdTuning))]
 
 
 class FwdGeometry(C.Structure):
@@ -151,6 +151,9 @@ SYMBOLS = {
     "pat_fwd_static_scratch_bytes": (C.c_size_t, []),
     "pat_fwd_slots_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_derive_slots": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_size_t, i64p, C.c_void_p]),
+    "pat_fwd_autotune_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
+    "pat_fwd_autotune": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_int32, C.c_void_p, C.c_size_t,
+                                   C.POINTER(FwdTuning), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "pat_fwd_set_tuning": (C.c_int, [C.POINTER(FwdTuning)]),
     "pat_fwd_get_tuning": (C.c_int, [C.POINTER(FwdTuning)]),
     "pat_paged_decode_baseline_workspace_bytes": (C.c_int, [C.POINTER(BaselineArgs), C.POINTER(C.c_size_t)]),

@@ -13,6 +13,7 @@
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
 #include <cstring>
 #include <memory>
@@ -72,8 +73,76 @@ struct Prepared {
   std::vector<pat_fwd_bucket> buckets;
   TensorList keep;          // plan tensors (and derived slots) stay alive as long as the launch does
   size_t need = 0;          // workspace bytes
-  Prepared() { std::memset(&args, 0, sizeof(args)); }
+  pat_fwd_tuning tuning;    // the measured geometry of this plan shape (args.tuning points here when set)
+  Prepared() { std::memset(&args, 0, sizeof(args)); std::memset(&tuning, 0, sizeof(tuning)); }
 };
+
+// ---- measured launch geometry, remembered per plan shape ---------------------------------------
+// pat_fwd_autotune times a launch under a few candidate geometries. One measurement serves every
+// launch of the same shape: the layers of a model call the forward with the same plan and
+// different caches, and consecutive decode steps differ by a token per request. The shape key
+// holds the head geometry and, per bucket, the tile label and the box count and block-table width
+// rounded up to multiples of 8.
+std::mutex g_tune_mutex;
+std::unordered_map<std::string, pat_fwd_tuning> g_tuned;
+bool g_autotune = [] {
+  const char* e = std::getenv("PAT_AUTOTUNE");
+  return e == nullptr || std::atoi(e) != 0;
+}();
+
+std::string shape_key(const pat_fwd_args& a) {
+  std::string k;
+  auto add = [&](int64_t v) { k.append(reinterpret_cast<const char*>(&v), sizeof(v)); };
+  auto up8 = [](int64_t v) { return (v + 7) / 8 * 8; };
+  add(a.dtype); add(a.head_dim); add(a.heads); add(a.kv_heads); add(a.page_size); add(up8(a.batch));
+  add(a.max_split_per_seq); add(a.num_buckets); add(a.lse_out != nullptr);
+  for (int i = 0; i < a.num_buckets; ++i) {
+    const pat_fwd_bucket& b = a.buckets[i];
+    add(b.mnw[0]); add(up8(b.num_boxes)); add(b.max_seqs); add(up8(b.max_blocks)); add(b.flags); add(b.q_slot != nullptr);
+  }
+  return k;
+}
+
+// Sets L.args.tuning from the remembered measurement of this shape, measuring first when there is
+// none (not while the stream is being captured into a graph: the measurement synchronises).
+void tune(Prepared& L, const c10::Device& dev) {
+  if (!g_autotune) return;
+  const std::string key = shape_key(L.args);
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    auto it = g_tuned.find(key);
+    if (it != g_tuned.end()) { L.tuning = it->second; L.args.tuning = &L.tuning; return; }
+  }
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  void* stream = static_cast<void*>(c10::hip::getCurrentHIPStream(dev.index()).stream());
+  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
+      capturing != hipStreamCaptureStatusNone)
+    return;
+  size_t most = 0;
+  check(pat_fwd_autotune_workspace_bytes(&L.args, &most));
+  at::Tensor ws = at::empty({(int64_t)std::max<size_t>(most, 256)}, at::TensorOptions().dtype(at::kByte).device(dev));
+  L.args.workspace = ws.data_ptr(); L.args.workspace_bytes = (size_t)ws.numel();
+  // 320 MB per device, read between the timed launches (more than the 256 MB memory-side cache holds):
+  // allocated at the first measurement and kept
+  static std::mutex evict_mutex;
+  static std::unordered_map<int, at::Tensor> evict_buffers;
+  at::Tensor evict;
+  {
+    std::lock_guard<std::mutex> lock(evict_mutex);
+    auto it = evict_buffers.find(dev.index());
+    if (it == evict_buffers.end())
+      it = evict_buffers.emplace(dev.index(), at::zeros({(int64_t)320 << 20}, at::TensorOptions().dtype(at::kByte).device(dev))).first;
+    evict = it->second;
+  }
+  pat_fwd_tuning best;
+  const int rc = pat_fwd_autotune(&L.args, stream, 8, evict.data_ptr(), (size_t)evict.numel(), &best, nullptr, nullptr);
+  L.args.workspace = nullptr; L.args.workspace_bytes = 0;
+  check(rc);
+  L.tuning = best; L.args.tuning = &L.tuning;
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  if (g_tuned.size() >= 4096) g_tuned.clear();
+  g_tuned[key] = best;
+}
 
 void strides3(const at::Tensor& t, int64_t out[3]) {
   out[0] = t.stride(0); out[1] = t.stride(1); out[2] = t.stride(2);
@@ -190,6 +259,7 @@ std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, cons
     a.num_split_per_seq = base;
     L->keep.push_back(derived);
   }
+  tune(*L, q.device());
   check(pat_fwd_workspace_bytes(&a, &L->need));
   return L;
 }
@@ -608,6 +678,16 @@ PYBIND11_MODULE(_prefix_attn, m) {
         }
         return out;
       })
+      .def_property_readonly("_launch_tunings", [](const KernelInfo& ki) {
+        std::vector<std::vector<int64_t>> out;   // per cached launch: the overrides in struct order, {} = none
+        for (const auto& kv : ki.cache) {
+          const pat_fwd_tuning& t = kv.second->tuning;
+          if (kv.second->args.tuning == nullptr) out.emplace_back();
+          else out.push_back({t.chunk_tokens, t.tall_chunk_tokens, t.head_per_wave_tokens, t.head_per_wave_long_tokens,
+                              t.head_per_wave_long_wgs, t.equalize_chunks, t.direct_out});
+        }
+        return out;
+      })
       .def_property_readonly("_launch_workspace_bytes", [](const KernelInfo& ki) {
         std::vector<size_t> out;
         for (const auto& kv : ki.cache) out.push_back(kv.second->need);
@@ -634,6 +714,12 @@ PYBIND11_MODULE(_prefix_attn, m) {
   m.def("prefix_attn_with_kvcache", &fwd_tree, py::arg("q"), py::arg("k_cache_paged"), py::arg("v_cache_paged"),
         py::arg("tree"), py::arg("softmax_scale"), py::arg("out"), py::kw_only(), py::arg("softmax_lse") = py::none(),
         "Tree form: the plan of a PrefixTreeCPP whose kernel_info is on the device.");
+  m.def("set_autotune", [](bool on) { g_autotune = on; }, py::arg("enabled"),
+        "Measured choice of the launch geometry (pat_fwd_autotune) the first time a plan shape is launched: on by "
+        "default (PAT_AUTOTUNE=0 in the environment switches it off). The measurement runs the launch a few "
+        "times per candidate on the current stream and synchronises it once per shape.");
+  m.def("get_autotune", [] { return g_autotune; });
+  m.def("clear_autotune_cache", [] { std::lock_guard<std::mutex> lock(g_tune_mutex); g_tuned.clear(); });
   m.def("paged_decode_baseline", &paged_decode_baseline, py::arg("q"), py::arg("k_cache_paged"),
         py::arg("v_cache_paged"), py::arg("block_table"), py::arg("seq_lens"), py::arg("softmax_scale"), py::arg("out"),
         py::arg("softmax_lse") = py::none(), py::arg("even_lengths") = false,

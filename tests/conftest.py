@@ -62,8 +62,11 @@ def tuning():
     """Sets launch-geometry overrides of libpat_amd (pat_fwd_set_tuning) for one test:
     `tuning(direct_out=0)`; the automatic values come back when the test ends."""
     import ctypes as C
-    from pat_amd import _lib
+    from pat_amd import _lib, _prefix_attn
     lib = _lib.load()
+    # the binding's measured geometry would take precedence over the process-wide overrides
+    measured = _prefix_attn.get_autotune()
+    _prefix_attn.set_autotune(False)
 
     def apply(**fields):
         t = _lib.FwdTuning.automatic()
@@ -75,3 +78,4 @@ def tuning():
     yield apply
     auto = _lib.FwdTuning.automatic()
     lib.pat_fwd_set_tuning(C.byref(auto))
+    _prefix_attn.set_autotune(measured)

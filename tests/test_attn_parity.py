@@ -725,3 +725,52 @@ def test_randomized_workloads_fixed_seed():
         ref_out, ref_lse = _oracle(w, q, k, v)
         _assert_close(f"random {done}", out, lse, ref_out, ref_lse, dtype)
         done += 1
+
+
+def test_autotuned_geometry_matches_oracle_and_is_remembered():
+    # the measured choice of the launch geometry: whichever candidate wins, the result is the
+    # oracle's; the C entry point reports a candidate that the launch accepts; the binding measures
+    # once per plan shape and reuses the choice for other tensors of the same plan
+    print("[case] autotune on c2: C entry point, then the drop-in call", flush=True)
+    import ctypes as C
+    from pat_amd import _ctypes_launch, _lib, _prefix_attn
+    dev = _device()
+    w = workloads.make("c2", seed=0)
+    q, ks, vs = w.tensors(dev, copies=2)
+    ref_out, ref_lse = _oracle(w, q, ks[0], vs[0])
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    lt = info.launch_tables()
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    L = _ctypes_launch.prepare(q, ks[0], vs[0], info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
+                               lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
+                               info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                               1.0 / math.sqrt(w.head_dim), out, lse, lt["slot_tables"], lt.get("flags"), autotune=True)
+    torch.cuda.synchronize()
+    print(f"        tuning run: chosen {L.tuned_us:.1f} us, automatic {L.auto_us:.1f} us, overrides "
+          f"{[getattr(L.tuning, f) for f, _ in _lib.FwdTuning._fields_]}", flush=True)
+    assert 0 < L.tuned_us <= L.auto_us
+    _assert_close("c2 after the tuning run", out, lse, ref_out, ref_lse, w.dtype)   # `out` is valid after tuning
+    out.fill_(float("nan")); lse.fill_(float("nan"))
+    _ctypes_launch.run(L, dev)
+    torch.cuda.synchronize()
+    _assert_close("c2 tuned launch", out, lse, ref_out, ref_lse, w.dtype)
+    # the drop-in call: measured on first use, remembered for the second cache
+    was = _prefix_attn.get_autotune()
+    _prefix_attn.set_autotune(True)
+    _prefix_attn.clear_autotune_cache()
+    try:
+        for i in range(2):
+            out.fill_(float("nan")); lse.fill_(float("nan"))
+            prefix_attn_with_kvcache(q, ks[i], vs[i], tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+            torch.cuda.synchronize()
+            if i == 0:
+                _assert_close("c2 drop-in call, tuned", out, lse, ref_out, ref_lse, w.dtype)
+        chosen = info._launch_tunings
+        assert len(chosen) == 2 and chosen[0] == chosen[1] and len(chosen[0]) == 7
+    finally:
+        _prefix_attn.set_autotune(was)
