@@ -459,7 +459,7 @@ int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, vo
   mp.o_part = o_part; mp.lse_part = lse_part; mp.num_split_per_seq = args->num_split_per_seq;
   mp.out = args->out; mp.lse_out = args->lse_out;
   mp.o_stride_b = args->o_stride[0]; mp.o_stride_h = args->o_stride[2];
-  mp.batch = args->batch; mp.heads = args->heads; mp.head_dim = args->head_dim;
+  mp.batch = args->batch; mp.heads = args->heads; mp.head_dim = args->head_dim; mp.kv_heads = args->kv_heads;
   mp.chunks_per_rank = g.chunks_per_rank; mp.num_slots = g.num_slots; mp.max_split = args->max_split_per_seq;
   const hipError_t e = launch_merge(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, mp);
   if (e != hipSuccess) return hip_fail(e, "merge kernel launch");

@@ -68,6 +68,7 @@ struct MergeParams {
   int64_t o_stride_b, o_stride_h;
   int32_t batch, heads, head_dim;
   int32_t chunks_per_rank, num_slots, max_split;
+  int32_t kv_heads;
 };
 
 }  // namespace pat

@@ -23,10 +23,27 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
   constexpr int kRegs = 4;      // LSE registers per lane: up to 256 slots stay in registers
   constexpr int kBatch = 16;    // partial rows fetched together
   const int lane = threadIdx.x & 63;
-  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (pair >= (int64_t)p.batch * p.heads) return;
-  const int s = (int)(pair / p.heads);
-  const int hq = (int)(pair % p.heads);
+  // Which (sequence, head) is this wave's? Workgroups are dealt to the 8 XCDs round-robin, and the
+  // split kernel's launch order put every partial row of kv head h through the L2 of XCD h mod 8
+  // (where most of it still sits): with a multiple of 8 kv heads, workgroup b serves heads of the kv
+  // heads = b mod 8, so the rows are found in its own L2. A matter of speed only.
+  int s, hq;
+  if (p.kv_heads % 8 == 0) {
+    const int xcd = blockIdx.x & 7;
+    const int per_seq = p.heads >> 3;                       // heads of one sequence served by one XCD
+    const int64_t u = (int64_t)(blockIdx.x >> 3) * 4 + (threadIdx.x >> 6);
+    if (u >= (int64_t)p.batch * per_seq) return;
+    s = (int)(u / per_seq);
+    const int local = (int)(u - (int64_t)s * per_seq);      // kv head (xcd + 8 i), head g of its group
+    const int group = p.heads / p.kv_heads;
+    hq = (xcd + 8 * (local / group)) * group + local % group;
+  } else {
+    const int64_t u = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (u >= (int64_t)p.batch * p.heads) return;
+    s = (int)(u / p.heads);
+    hq = (int)(u % p.heads);
+  }
+  const int64_t pair = (int64_t)s * p.heads + hq;
   const float ninf = -__builtin_inff();
 
   const float* __restrict__ lse = p.lse_part + pair * p.num_slots;
@@ -116,7 +133,9 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
 // Host launcher: one wave per (sequence, query head), four per workgroup.
 hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params) {
   const int64_t pairs = (int64_t)params.batch * params.heads;
-  const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
+  // (a multiple of 8 kv heads: 8 interleaved lists of pairs, one per XCD, each rounded up to whole workgroups)
+  const int64_t wgs = params.kv_heads % 8 == 0 ? 8 * ((pairs / 8 + 3) / 4) : (pairs + 3) / 4;
+  const dim3 grid((unsigned)wgs), block(256);
   void (*fn)(const MergeParams);
   if (bf16) fn = head_dim == 64 ? pat_merge_kernel<__bf16, 64> : pat_merge_kernel<__bf16, 128>;
   else fn = head_dim == 64 ? pat_merge_kernel<_Float16, 64> : pat_merge_kernel<_Float16, 128>;

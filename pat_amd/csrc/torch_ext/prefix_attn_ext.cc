@@ -95,7 +95,7 @@ std::string shape_key(const pat_fwd_args& a) {
   auto add = [&](int64_t v) { k.append(reinterpret_cast<const char*>(&v), sizeof(v)); };
   auto up8 = [](int64_t v) { return (v + 7) / 8 * 8; };
   add(a.dtype); add(a.head_dim); add(a.heads); add(a.kv_heads); add(a.page_size); add(up8(a.batch));
-  add(a.max_split_per_seq); add(a.num_buckets); add(a.lse_out != nullptr);
+  add(a.max_split_per_seq); add(a.num_buckets);   // (not whether an LSE is asked for: one call's geometry serves both)
   for (int i = 0; i < a.num_buckets; ++i) {
     const pat_fwd_bucket& b = a.buckets[i];
     add(b.mnw[0]); add(up8(b.num_boxes)); add(b.max_seqs); add(up8(b.max_blocks)); add(b.flags); add(b.q_slot != nullptr);
