@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PAT_ABI_VERSION 2
+#define PAT_ABI_VERSION 3
 
 /* ---- status codes ------------------------------------------------------- */
 #define PAT_OK 0
@@ -294,6 +294,9 @@ typedef struct pat_fwd_args {
                                  /* split kernel and the merge kernel (timing aid), or NULL  */
   const pat_fwd_tuning* tuning;  /* optional launch-geometry overrides for this call (host    */
                                  /* memory, read during the call); NULL: the process-wide ones */
+  const void* records;           /* optional launch records of this plan (pat_fwd_build_records), */
+  size_t records_bytes;          /* device memory; NULL: the launch builds them in its workspace  */
+  uint64_t records_tag;          /* what pat_fwd_build_records returned with them                 */
 } pat_fwd_args;
 
 /* Argument checks of csrc/api.h:129-181 that need no GPU (dtype enum, head_dim,
@@ -301,13 +304,35 @@ typedef struct pat_fwd_args {
  * tested for NULL. Runs on a machine without a GPU. */
 int pat_fwd_validate(const pat_fwd_args* args);
 
-/* Bytes of device scratch pat_fwd_launch needs for these arguments (partial
- * outputs + partial LSE; the reference allocates the equivalent per call at
- * csrc/api.h:217-229). Depends only on sizes, pointers' alignment and strides, never on
- * device data. 0 when every row has a single partial slot (max_split_per_seq 1 and no box
- * longer than a chunk): the launch then writes `out` from its first kernel, as the reference
- * does for max_split_per_seq 1 (csrc/api.h:230-238), and `workspace` may be NULL. */
+/* Bytes of device scratch pat_fwd_launch needs for these arguments: partial outputs +
+ * partial LSE (the reference allocates the equivalent per call at csrc/api.h:217-229) and,
+ * when args->records is NULL, the launch records of this call. Depends only on sizes,
+ * pointers' alignment and strides, never on device data. With prebuilt records it is 0 when
+ * every row has a single partial slot (max_split_per_seq 1 and no box longer than a chunk):
+ * the launch then writes `out` from its first kernel, as the reference does for
+ * max_split_per_seq 1 (csrc/api.h:230-238), and `workspace` may be NULL. */
 int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes);
+
+/* Launch records: one small record per workgroup of the launch (which rows, which partial
+ * slots, which KV pages, how many tokens), laid out so that the split kernel starts its KV
+ * loads after a single round trip to memory. A device kernel writes them from the plan tables
+ * (values checked and clamped there once, not in every launch). They depend on the plan tables'
+ * contents, on the sizes in `args` and on the launch geometry (tuning), not on q / k / v / out:
+ * build them once per plan and pass them to every launch of it (each layer of a decode step);
+ * rebuild after the plan tables were edited. pat_fwd_launch with args->records == NULL builds
+ * them itself on every call, in its workspace (one more small kernel per call).
+ * No counterpart in the reference, whose kernel decodes the plan tables in every thread block
+ * (csrc/pat_fwd_kernel.h:40-75).
+ * pat_fwd_records_bytes: size of the buffer; pat_fwd_build_records: enqueues the record kernel
+ * on `hip_stream` (`buffer`: device memory, 256-byte aligned) and returns the tag to put in
+ * args->records_tag; a launch whose geometry or tables differ from the tag's fails with
+ * PAT_ERR_INVALID and enqueues nothing. pat_fwd_records_tag: the tag alone (host arithmetic): two
+ * argument blocks with the same tag can share one set of records (the layers of a model: same
+ * plan tables, different q / k / v / out). */
+int pat_fwd_records_bytes(const pat_fwd_args* args, size_t* bytes);
+int pat_fwd_records_tag(const pat_fwd_args* args, uint64_t* tag);
+int pat_fwd_build_records(const pat_fwd_args* args, void* buffer, size_t buffer_bytes,
+                          uint64_t* tag, void* hip_stream);
 
 /* prefix_attn_with_kvcache(...)   csrc/bindings.cpp:7-72 -> csrc/api.h:110-295
  * Enqueues the split-KV kernel and (unless the workspace size is 0, see above) the merge

@@ -33,7 +33,8 @@ class _Launch:
 
 
 def prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MNW, max_split,
-            max_seqs, max_blocks, scale, out, lse, slot_tables=None, bucket_flags=None, autotune=False, tuning=None) -> _Launch:
+            max_seqs, max_blocks, scale, out, lse, slot_tables=None, bucket_flags=None, autotune=False, tuning=None,
+            build_records=True) -> _Launch:
     lib = _lib.load()
     # --- checks that need tensor metadata (csrc/api.h:131-181, :256-277) -----------------
     _check(q.dtype in (torch.float16, torch.bfloat16), "only support fp16 and bf16 data type")
@@ -135,13 +136,23 @@ def prepare(q, k, v, num_split, q_tables, block_tables, num_seqs, ranks, kvs, MN
         a.tuning = C.pointer(L.tuning)
         a.workspace, a.workspace_bytes = None, 0
         L.tuned_us, L.auto_us = best_us.value, auto_us.value
+    records = None
+    if build_records:
+        # the launch records of this plan under the geometry just chosen: one small kernel now,
+        # none in the launches
+        rbytes, tag = C.c_size_t(0), C.c_uint64(0)
+        _lib.check(lib.pat_fwd_records_bytes(C.byref(a), C.byref(rbytes)))
+        records = torch.empty(rbytes.value, dtype=torch.uint8, device=q.device)
+        _lib.check(lib.pat_fwd_build_records(C.byref(a), C.c_void_p(records.data_ptr()), rbytes.value, C.byref(tag),
+                                             C.c_void_p(_raw_stream(q.device.index))))
+        a.records, a.records_bytes, a.records_tag = records.data_ptr(), rbytes.value, tag.value
     need = C.c_size_t(0)
     _lib.check(lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)))
     L.args, L.need = a, need.value
     # plan tensors stay referenced as long as the prepared launch does; q/k/v/out are the
     # caller's for the duration of the call only
     L.keep = (num_split, list(q_tables), list(block_tables), list(num_seqs), list(ranks), list(kvs),
-              None if slot_tables is None else list(slot_tables), derived)
+              None if slot_tables is None else list(slot_tables), derived, records)
     L.workspace = None
     return L
 

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpat_amd.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 PAT_OK = 0
 PAT_ERR_INVALID = -1
@@ -120,7 +120,8 @@ class FwdArgs(C.Structure):
                 ("max_blocks_in_box", C.c_int32), ("softmax_scale", C.c_float),
                 ("num_buckets", C.c_int32), ("buckets", C.POINTER(FwdBucket)),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-                ("split_done_event", C.c_void_p), ("tuning", C.POINTER(FwdTuning))]
+                ("split_done_event", C.c_void_p), ("tuning", C.POINTER(FwdTuning)),
+                ("records", C.c_void_p), ("records_bytes", C.c_size_t), ("records_tag", C.c_uint64)]
 
 
 class FwdGeometry(C.Structure):
@@ -151,6 +152,9 @@ SYMBOLS = {
     "pat_fwd_static_scratch_bytes": (C.c_size_t, []),
     "pat_fwd_slots_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_derive_slots": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_size_t, i64p, C.c_void_p]),
+    "pat_fwd_records_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
+    "pat_fwd_records_tag": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_uint64)]),
+    "pat_fwd_build_records": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_size_t, C.POINTER(C.c_uint64), C.c_void_p]),
     "pat_fwd_autotune_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),
     "pat_fwd_autotune": (C.c_int, [C.POINTER(FwdArgs), C.c_void_p, C.c_int32, C.c_void_p, C.c_size_t,
                                    C.POINTER(FwdTuning), C.POINTER(C.c_float), C.POINTER(C.c_float)]),

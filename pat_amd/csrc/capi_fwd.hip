@@ -82,6 +82,8 @@ struct Geometry {
   int bucket_heads_per_wg[kMaxBuckets] = {0};   // 1, or kWaves: one kv head per wave
   int64_t total_wgs = 0;
   bool direct = false;       // one slot per row: the split kernel writes `out`, no workspace, no merge kernel
+  // launch records (one per workgroup): entries per record and bytes between records
+  int record_max_seqs = 0, record_max_pages = 0, record_stride = 0;
 };
 
 int check_args(const pat_fwd_args* a) {
@@ -332,6 +334,14 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
               a->o_stride[2] % 4 == 0 && tune.direct_out != 0;
   if (g->total_wgs > (int64_t)kGridX * 65535 || g->total_wgs >= INT32_MAX)
     return fail(PAT_ERR_INVALID, "too many workgroups for one launch");
+  for (int i = 0; i < a->num_buckets; ++i) {
+    if (a->buckets[i].num_boxes == 0) continue;
+    g->record_max_seqs = std::max(g->record_max_seqs, (int)a->buckets[i].max_seqs);
+    g->record_max_pages = std::max(g->record_max_pages, (int)ceil_div64(g->bucket_chunk[i], page));
+  }
+  g->record_max_seqs = std::min(std::max(g->record_max_seqs, 1), 64);
+  g->record_max_pages = std::min(std::max(g->record_max_pages, 1), kMaxChunkPages);
+  g->record_stride = (int)((sizeof(RecordHead) + (2 * g->record_max_seqs + g->record_max_pages) * sizeof(int32_t) + 63) / 64 * 64);
   // the kernels index partial rows with 32-bit integers
   if ((int64_t)a->batch * a->heads * g->num_slots >= ((int64_t)1 << 31))
     return fail(PAT_ERR_INVALID, "batch * heads * partial slots must stay below 2^31");
@@ -340,10 +350,37 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t workspace_need(const pat_fwd_args* a, const Geometry& g) {
+size_t partials_need(const pat_fwd_args* a, const Geometry& g) {
   if (g.direct) return 0;
   const size_t rows = (size_t)a->batch * a->heads * g.num_slots;
   return align256(rows * a->head_dim * sizeof(float)) + align256(rows * sizeof(float));
+}
+// (records for the whole grid: beyond kGridX workgroups the grid is padded to whole slices)
+int64_t grid_wgs(const Geometry& g) { return g.total_wgs <= kGridX ? g.total_wgs : ceil_div64(g.total_wgs, kGridX) * kGridX; }
+size_t records_need(const Geometry& g) { return align256((size_t)grid_wgs(g) * (size_t)g.record_stride); }
+// The workspace of a launch: the partial results, then - when the caller did not build the launch
+// records beforehand (pat_fwd_build_records) - the records of this call.
+size_t workspace_need(const pat_fwd_args* a, const Geometry& g) {
+  return partials_need(a, g) + (a->records == nullptr ? records_need(g) : 0);
+}
+
+// What a set of launch records depends on besides the contents of the plan tables: the geometry
+// and the tables' addresses and sizes. pat_fwd_build_records hands it out, launches compare.
+uint64_t records_tag(const pat_fwd_args* a, const Geometry& g) {
+  uint64_t h = 0x9e3779b97f4a7c15ull;
+  auto mix = [&](uint64_t v) { h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2); };
+  mix((uint64_t)g.total_wgs); mix((uint64_t)g.record_stride); mix((uint64_t)g.record_max_seqs); mix((uint64_t)g.record_max_pages);
+  mix((uint64_t)g.num_slots); mix((uint64_t)g.chunks_per_rank); mix(g.direct ? 1 : 0);
+  mix((uint64_t)a->batch); mix((uint64_t)a->heads); mix((uint64_t)a->kv_heads); mix((uint64_t)a->page_size);
+  mix((uint64_t)a->num_pages); mix((uint64_t)a->max_split_per_seq);
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const pat_fwd_bucket& b = a->buckets[i];
+    mix((uint64_t)g.bucket_chunk[i]); mix((uint64_t)g.bucket_chunks[i]); mix((uint64_t)g.bucket_heads_per_wg[i]);
+    mix((uint64_t)b.num_boxes); mix((uint64_t)b.max_seqs); mix((uint64_t)b.max_blocks); mix((uint64_t)b.mnw[0]);
+    mix((uint64_t)reinterpret_cast<uintptr_t>(b.q_table)); mix((uint64_t)reinterpret_cast<uintptr_t>(b.block_table));
+    mix((uint64_t)reinterpret_cast<uintptr_t>(b.kv)); mix((uint64_t)reinterpret_cast<uintptr_t>(b.q_slot));
+  }
+  return h ? h : 1;
 }
 
 int hip_fail(hipError_t e, const char* what) {
@@ -385,7 +422,123 @@ int pat_fwd_workspace_bytes(const pat_fwd_args* args, size_t* bytes) {
 namespace pat {
 namespace {
 
-// Everything pat_fwd_launch does after the argument checks: `workspace` holds the partial results.
+// ---- launch records ------------------------------------------------------------------------------
+// One wave per record: decodes which (bucket, box, chunk, kv head group) the workgroup is, reads
+// the box's plan entries, checks and clamps them, and lays them out for the split kernel.
+__global__ void __launch_bounds__(256) pat_record_kernel(const RecordParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wg = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wg >= p.grid_items) return;
+  if (wg >= p.total_items) {
+    // padding of the grid: a workgroup with nothing to do
+    char* rec = p.records + (size_t)wg * (size_t)p.record_stride;
+    int32_t* words = reinterpret_cast<int32_t*>(rec);
+    for (int i = lane; i < p.record_stride / 4; i += 64) words[i] = (i < 8) ? 0 : -1;
+    return;
+  }
+  int bi = 0;
+  for (int i = 1; i < p.num_buckets; ++i) bi += (wg >= p.bucket[i].item_begin) ? 1 : 0;
+  const RecordBucket bk = p.bucket[bi];
+  const int head_groups = p.kv_heads / bk.heads_per_wg;
+  const int wg_local = wg - bk.item_begin;
+  const int local = wg_local / head_groups;
+  const int hgroup = wg_local - local * head_groups;
+  // chunk-major inside a bucket: all boxes' first chunks, then all second chunks, ... Workgroups
+  // are handed to the shader engines round-robin in launch order and the hand-out stalls while
+  // the engine whose turn it is is full, so work must not correlate with the launch index: in
+  // box-major order the filled chunks of short boxes recur with the period of the reserved
+  // chunks, land on the same engines every time and leave the others idle.
+  const int chunk = local / bk.num_boxes;
+  const int box = local - chunk * bk.num_boxes;
+  const int page = p.page_size;
+  int nseq = bk.num_seqs[box];
+  nseq = nseq < 0 ? 0 : (nseq > bk.max_seqs ? bk.max_seqs : nseq);
+  int rows = nseq * p.group;
+  if (rows > 16 * bk.row_tiles) rows = 16 * bk.row_tiles;
+  int kv = bk.kv[box];
+  const int kv_cap = bk.max_blocks * page;
+  kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
+  const int t_begin = chunk * bk.chunk_tokens;
+  int tokens = kv - t_begin;
+  tokens = tokens < 0 ? 0 : (tokens > bk.chunk_tokens ? bk.chunk_tokens : tokens);
+  const int rank = bk.rank[box];
+
+  char* rec = p.records + (size_t)wg * (size_t)p.record_stride;
+  if (lane == 0) {
+    RecordHead h;
+    h.tokens = rows > 0 ? tokens : 0;
+    h.rows = rows;
+    h.mode = bk.row_tiles | (bk.heads_per_wg > 1 ? kRecordModeHeadPerWave : 0);
+    h.head = hgroup * bk.heads_per_wg;
+    // slots of this box that no workgroup fills: this one's own when it has no tokens, and the
+    // ones past the bucket's last chunk (the launch reserves chunks_per_rank per box ordinal)
+    h.fill_begin = tokens > 0 ? 1 : 0;
+    h.fill_end = (chunk == bk.chunks - 1) ? p.chunks_per_rank - chunk : 1;
+    h.pad[0] = h.pad[1] = 0;
+    *reinterpret_cast<RecordHead*>(rec) = h;
+  }
+  int32_t* tab = reinterpret_cast<int32_t*>(rec + sizeof(RecordHead));
+  // rows: sequence id and partial-result slot (the plan's own rank or, when the plan carries
+  // them, the box's ordinal among the boxes of that sequence)
+  for (int j = lane; j < p.record_max_seqs; j += 64) {
+    int seq = -1, slot = -1;
+    if (j < nseq && j * p.group < rows) {
+      const int q = bk.q_table[(int64_t)box * bk.q_stride + j];
+      if ((unsigned)q < (unsigned)p.batch) seq = q;
+      const int ord = bk.q_slot ? bk.q_slot[(int64_t)box * bk.q_stride + j] : rank;
+      if ((unsigned)ord < (unsigned)p.max_split) slot = ord * p.chunks_per_rank + chunk;
+    }
+    tab[j] = seq;
+    tab[p.record_max_seqs + j] = slot;
+  }
+  // pages of the piece
+  const int first_page = t_begin / page;
+  for (int i = lane; i < p.record_max_pages; i += 64) {
+    int pg = (first_page + i < bk.max_blocks) ? bk.block_table[(int64_t)box * bk.bt_stride + first_page + i] : 0;
+    pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
+    tab[2 * p.record_max_seqs + i] = pg;
+  }
+}
+
+int build_records(const pat_fwd_args* args, const Geometry& g, void* buffer, hipStream_t stream) {
+  RecordParams rp;
+  std::memset(&rp, 0, sizeof(rp));
+  rp.records = static_cast<char*>(buffer);
+  rp.record_stride = g.record_stride; rp.record_max_seqs = g.record_max_seqs; rp.record_max_pages = g.record_max_pages;
+  rp.batch = args->batch; rp.kv_heads = args->kv_heads; rp.group = args->heads / args->kv_heads;
+  rp.page_size = args->page_size; rp.num_pages = args->num_pages;
+  rp.chunks_per_rank = g.chunks_per_rank; rp.max_split = args->max_split_per_seq;
+  // buckets in plan order (tall, long boxes come first in the default order)
+  int nb = 0;
+  int64_t items = 0;
+  for (int i = 0; i < args->num_buckets; ++i) {
+    const pat_fwd_bucket& b = args->buckets[i];
+    if (b.num_boxes == 0) continue;
+    RecordBucket& d = rp.bucket[nb];
+    d.q_table = b.q_table; d.block_table = b.block_table; d.num_seqs = b.num_seqs;
+    d.rank = b.rank; d.kv = b.kv; d.q_slot = b.q_slot;
+    d.q_stride = (int32_t)b.q_table_stride; d.bt_stride = (int32_t)b.block_table_stride;
+    d.num_boxes = b.num_boxes; d.max_seqs = b.max_seqs; d.max_blocks = b.max_blocks;
+    d.chunk_tokens = g.bucket_chunk[i];
+    d.chunks = g.bucket_chunks[i];
+    d.row_tiles = row_tiles(b.mnw[0]);
+    d.heads_per_wg = g.bucket_heads_per_wg[i];
+    d.item_begin = (int32_t)items;
+    ++nb;
+    items += (int64_t)b.num_boxes * d.chunks * (args->kv_heads / d.heads_per_wg);
+  }
+  if (items != g.total_wgs) return fail(PAT_ERR_INVALID, "internal: workgroup count of the records differs from the geometry");
+  rp.num_buckets = nb;
+  rp.total_items = (int32_t)items;
+  rp.grid_items = (int32_t)grid_wgs(g);
+  if (items == 0) return PAT_OK;
+  hipLaunchKernelGGL(pat_record_kernel, dim3((unsigned)((rp.grid_items + 3) / 4)), dim3(256), 0, stream, rp);
+  if (const hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "record kernel launch");
+  return PAT_OK;
+}
+
+// Everything pat_fwd_launch does after the argument checks: `workspace` holds the partial results
+// and, behind them, the launch records when the caller brought none.
 int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, void* hip_stream) {
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
 
@@ -393,9 +546,21 @@ int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, vo
   float* o_part = static_cast<float*>(workspace);
   float* lse_part = reinterpret_cast<float*>(static_cast<char*>(workspace) +
                                              align256(rows * args->head_dim * sizeof(float)));
+  const void* records = args->records;
+  if (records != nullptr) {
+    if (args->records_tag != records_tag(args, g))
+      return fail(PAT_ERR_INVALID, "launch records were built for another plan or launch geometry");
+    if (args->records_bytes < records_need(g)) return fail(PAT_ERR_INVALID, "launch records: buffer smaller than the launch needs");
+  } else if (g.total_wgs > 0) {
+    void* own = static_cast<char*>(workspace) + partials_need(args, g);
+    if (int rc = build_records(args, g, own, stream)) return rc;
+    records = own;
+  }
 
   SplitParams sp;
   std::memset(&sp, 0, sizeof(sp));
+  sp.records = static_cast<const char*>(records);
+  sp.record_stride = g.record_stride; sp.record_max_seqs = g.record_max_seqs;
   sp.q = args->q; sp.k = args->k; sp.v = args->v;
   sp.o_part = o_part; sp.lse_part = lse_part;
   sp.direct = g.direct ? 1 : 0;
@@ -406,45 +571,19 @@ int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, vo
   sp.q_stride_b = args->q_stride[0]; sp.q_stride_h = args->q_stride[2];
   sp.k_stride_page = args->k_stride[0]; sp.k_stride_slot = args->k_stride[1]; sp.k_stride_h = args->k_stride[2];
   sp.v_stride_page = args->v_stride[0]; sp.v_stride_slot = args->v_stride[1]; sp.v_stride_h = args->v_stride[2];
-  sp.batch = args->batch; sp.heads = args->heads; sp.kv_heads = args->kv_heads;
+  sp.heads = args->heads;
   sp.group = args->heads / args->kv_heads;
-  sp.page_size = args->page_size; sp.num_pages = args->num_pages;
-  sp.chunks_per_rank = g.chunks_per_rank; sp.num_slots = g.num_slots;
+  sp.page_size = args->page_size;
+  sp.num_slots = g.num_slots;
   {
     const uint64_t hpp = (uint64_t)args->page_size / 16;
     sp.hpp_magic = hpp > 1 ? (uint32_t)((((uint64_t)1 << 32) + hpp - 1) / hpp) : 0u;
   }
-  sp.max_split = args->max_split_per_seq;
   sp.scale_log2 = args->softmax_scale * 1.4426950408889634f;
-
-  // one launch over all buckets, in plan order (tall, long boxes come first in the default order)
-  {
-    int nb = 0;
-    int64_t items = 0;
-    for (int i = 0; i < kMaxBuckets; ++i) sp.item_begin[i] = INT32_MAX;
-    for (int i = 0; i < args->num_buckets; ++i) {
-      const pat_fwd_bucket& b = args->buckets[i];
-      if (b.num_boxes == 0) continue;
-      BucketDev& d = sp.bucket[nb];
-      d.q_table = b.q_table; d.block_table = b.block_table; d.num_seqs = b.num_seqs;
-      d.rank = b.rank; d.kv = b.kv; d.q_slot = b.q_slot;
-      d.q_stride = (int32_t)b.q_table_stride; d.bt_stride = (int32_t)b.block_table_stride;
-      d.num_boxes = b.num_boxes; d.max_seqs = b.max_seqs; d.max_blocks = b.max_blocks;
-      d.chunk_tokens = g.bucket_chunk[i];
-      d.chunks = g.bucket_chunks[i];
-      d.row_tiles = row_tiles(b.mnw[0]);
-      d.heads_per_wg = g.bucket_heads_per_wg[i];
-      d.item_begin = (int32_t)items;
-      sp.item_begin[nb] = (int32_t)items;
-      ++nb;
-      items += (int64_t)b.num_boxes * d.chunks * (args->kv_heads / d.heads_per_wg);
-    }
-    sp.num_buckets = nb;
-    sp.total_items = (int32_t)items;
-    if (items > 0) {
-      const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, sp);
-      if (e != hipSuccess) return hip_fail(e, "split kernel launch");
-    }
+  sp.total_items = (int32_t)g.total_wgs;
+  if (g.total_wgs > 0) {
+    const hipError_t e = launch_split(args->dtype == PAT_DTYPE_BF16, args->head_dim, stream, sp);
+    if (e != hipSuccess) return hip_fail(e, "split kernel launch");
   }
 
   if (args->split_done_event != nullptr) {
@@ -534,7 +673,44 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream) {
                                        std::to_string(args->workspace_bytes));
   if (need > 0 && reinterpret_cast<uintptr_t>(args->workspace) % 256 != 0)
     return fail(PAT_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  if (args->records != nullptr && reinterpret_cast<uintptr_t>(args->records) % 256 != 0)
+    return fail(PAT_ERR_WORKSPACE, "launch records must be 256-byte aligned");
   return launch_core(args, g, args->workspace, hip_stream);
+}
+
+int pat_fwd_records_bytes(const pat_fwd_args* args, size_t* bytes) {
+  using namespace pat;
+  if (bytes == nullptr) return fail(PAT_ERR_INVALID, "bytes is NULL");
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  *bytes = std::max<size_t>(records_need(g), 256);
+  return PAT_OK;
+}
+
+int pat_fwd_records_tag(const pat_fwd_args* args, uint64_t* tag) {
+  using namespace pat;
+  if (tag == nullptr) return fail(PAT_ERR_INVALID, "tag is NULL");
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  *tag = records_tag(args, g);
+  return PAT_OK;
+}
+
+int pat_fwd_build_records(const pat_fwd_args* args, void* buffer, size_t buffer_bytes, uint64_t* tag, void* hip_stream) {
+  using namespace pat;
+  if (buffer == nullptr || tag == nullptr) return fail(PAT_ERR_INVALID, "buffer / tag is NULL");
+  if (int rc = check_args(args)) return rc;
+  Geometry g;
+  if (int rc = plan_geometry(args, &g)) return rc;
+  if (buffer_bytes < records_need(g))
+    return fail(PAT_ERR_WORKSPACE, "record buffer too small: need " + std::to_string(records_need(g)) + " bytes, got " +
+                                       std::to_string(buffer_bytes));
+  if (reinterpret_cast<uintptr_t>(buffer) % 256 != 0) return fail(PAT_ERR_WORKSPACE, "record buffer must be 256-byte aligned");
+  if (int rc = build_records(args, g, buffer, static_cast<hipStream_t>(hip_stream))) return rc;
+  *tag = records_tag(args, g);
+  return PAT_OK;
 }
 
 size_t pat_fwd_static_scratch_bytes(void) { return pat::kStaticScratchBytes; }
@@ -651,6 +827,7 @@ int pat_fwd_autotune_workspace_bytes(const pat_fwd_args* args, size_t* bytes) {
   for (int i = 0; i < n; ++i) {
     pat_fwd_args a = *args;
     a.tuning = &cand[i];
+    a.records = nullptr;
     Geometry g;
     if (plan_geometry(&a, &g) != PAT_OK) continue;   // a candidate this launch cannot take
     most = std::max(most, workspace_need(&a, g));
@@ -691,9 +868,16 @@ int pat_fwd_autotune(const pat_fwd_args* args, void* hip_stream, int32_t reps, c
     pat_fwd_args a = *args;
     a.tuning = &cand[i];
     a.split_done_event = nullptr;
+    a.records = nullptr;
     Geometry g;
     if (plan_geometry(&a, &g) != PAT_OK) continue;
     if (workspace_need(&a, g) > args->workspace_bytes) continue;   // (the automatic one always fits a sized workspace)
+    if (args->workspace == nullptr) { rc = fail(PAT_ERR_WORKSPACE, "pat_fwd_autotune needs a workspace"); break; }
+    // the candidate's launch records, built once behind its partial results: the timed launches are the two kernels only
+    void* rec = static_cast<char*>(args->workspace) + partials_need(&a, g);
+    rc = build_records(&a, g, rec, stream);
+    if (rc != PAT_OK) break;
+    a.records = rec; a.records_bytes = records_need(g); a.records_tag = records_tag(&a, g);
     for (int r = 0; r < 2 && rc == PAT_OK; ++r) rc = pat_fwd_launch(&a, hip_stream);
     if (rc != PAT_OK) break;
     hipError_t e = hipSuccess;
@@ -736,10 +920,11 @@ int pat_fwd_autotune(const pat_fwd_args* args, void* hip_stream, int32_t reps, c
   *best = cand[pick];
   if (best_us != nullptr) *best_us = us[pick];
   if (auto_us != nullptr) *auto_us = us[0];
-  if (pick != 0) {   // leave `out` as the chosen geometry computes it
+  if (pick != n - 1) {   // leave `out` as the chosen geometry computes it (the last candidate timed is in it now)
     pat_fwd_args a = *args;
     a.tuning = &cand[pick];
     a.split_done_event = nullptr;
+    a.records = nullptr;
     rc = pat_fwd_launch(&a, hip_stream);
   }
   return rc;

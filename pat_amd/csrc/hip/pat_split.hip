@@ -74,7 +74,8 @@ __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 #endif
 // DIRECT instances serve launches in which every row has one partial slot: they store `out`.
 template <typename T, int D, bool DIRECT>
-__global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const SplitParams p) {
+__global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const char* __restrict__ records, const int record_stride,
+                                                                  const int record_max_seqs, const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   constexpr int KK = D / 32;             // MFMA k-steps across head_dim in S^T = K.Q^T
@@ -105,83 +106,68 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const int g = lane >> 4;   // lane group 0..3
   const int n = lane & 15;   // index inside the group
 
-  // ---- which (bucket, box, chunk, kv-head) is this workgroup? ---------------------------
-  // a flat list of workgroups, head (group) fastest inside an item.
-  // The bucket is found from a table at fixed kernel-argument offsets and its descriptor is
-  // fetched whole, so the decode costs two scalar-memory round trips, not one per field.
-  const int wg_id = blockIdx.y * kGridX + blockIdx.x;   // past the last workgroup: lands past the last box
-  int bi = 0;
-#pragma unroll
-  for (int i = 1; i < kMaxBuckets; ++i) bi += (wg_id >= p.item_begin[i]) ? 1 : 0;
-  const BucketDev bk = p.bucket[bi];
-  // head group fastest: consecutive workgroups (dealt to the XCDs round-robin) serve consecutive
-  // kv heads of one item. Buckets of very short boxes give each wave a kv head of its own.
-  const bool head_per_wave = bk.heads_per_wg > 1;
-  const int head_groups = p.kv_heads / bk.heads_per_wg;
-  const int wg_local = wg_id - bk.item_begin;
-  const int local = wg_local / head_groups;
-  // (uniform over the wave: kept in a scalar register so that address arithmetic stays scalar)
-  const int head = __builtin_amdgcn_readfirstlane(
-      (wg_local - local * head_groups) * bk.heads_per_wg + (head_per_wave ? (int)(threadIdx.x >> 6) : 0));
-  // chunk-major inside a bucket: all boxes' first chunks, then all second chunks, ... Workgroups
-  // are handed to the shader engines round-robin in launch order and the hand-out stalls while
-  // the engine whose turn it is is full, so work must not correlate with the launch index: in
-  // box-major order the filled chunks of short boxes recur with the period of the reserved
-  // chunks, land on the same engines every time and leave the others idle.
-  const int chunk = local / bk.num_boxes;
-  const int box = local - chunk * bk.num_boxes;
-  if (chunk >= bk.chunks) return;
-
-  // Boxes of up to 16 rows: the 4 waves split the chunk's steps, each on wave-private tiles.
+  // ---- this workgroup's launch record: one round trip for everything the plan says about it ---
+  // (header, sequence ids and partial-result slots of its rows, page ids of its piece: checked,
+  // clamped and laid out by the record kernel once per plan). The launch is a flat list of
+  // workgroups; consecutive ones serve consecutive kv heads of one piece (workgroups are dealt to
+  // the 8 XCDs round-robin, so with 8 kv heads XCD x serves head x and the boxes that share KV
+  // pages find them in that XCD's L2), and inside a bucket the list is chunk-major.
+  // (the grid is padded to whole slices of kGridX only beyond 2^20 workgroups; the padding has
+  // records too, empty ones, so nothing here waits for a bound from the kernel arguments)
+  const unsigned wg_id = blockIdx.y * (unsigned)kGridX + blockIdx.x;
+  const char* __restrict__ rec = records + (size_t)wg_id * (unsigned)record_stride;
+  const int4 rh0 = *(const int4*)rec;
+  const int4 rh1 = *(const int4*)(rec + 16);
+  // The piece's length, twice: as a scalar for the loops of the shared-tile path, and laundered
+  // into a vector register for the wave-private path. With loop bounds it can prove uniform the
+  // compiler schedules the wave-private loops for 50 more registers (~200 spilled VGPRs at
+  // head_dim 128 under the 3-workgroups-per-CU budget); with vector bounds in the shared-tile path
+  // its per-step branches turn into masked execution of both sides (a step 20 % slower).
+  int ntok_v = rh0.x;
+  asm volatile("" : "+v"(ntok_v));
+  const int ntok = ntok_v;
+  const int ntok_u = __builtin_amdgcn_readfirstlane(rh0.x);
+  const int nsteps_u = (ntok_u + kStepTokens - 1) / kStepTokens;
+  const int R = __builtin_amdgcn_readfirstlane(rh0.y);
+  const int mode = __builtin_amdgcn_readfirstlane(rh0.z);
+  const bool head_per_wave = (mode & kRecordModeHeadPerWave) != 0;
+  // Boxes of up to 16 rows: the 4 waves split the piece's steps, each on wave-private tiles (or,
+  // with a kv head per wave, each wave walks all steps of its own head).
   // Taller boxes: wave w owns rows 16w..16w+15, all waves walk the same steps on tiles shared
   // through LDS.
-  const bool shared_tiles = bk.row_tiles > 1;
+  const bool shared_tiles = (mode & 0xff) > 1;
+  // (uniform over the wave: kept in a scalar register so that address arithmetic stays scalar)
+  const int head = __builtin_amdgcn_readfirstlane(rh0.w + (head_per_wave ? (int)(threadIdx.x >> 6) : 0));
+  const int fill_begin = __builtin_amdgcn_readfirstlane(rh1.x);
+  const int fill_end = __builtin_amdgcn_readfirstlane(rh1.y);
   const int G = p.group;
   const int page = p.page_size;
   const int row0 = shared_tiles ? wave * 16 : 0;
-  const int t_begin = chunk * bk.chunk_tokens;
-  const int* __restrict__ qt = bk.q_table + (int64_t)box * bk.q_stride;
-  const int* __restrict__ qs = bk.q_slot ? bk.q_slot + (int64_t)box * bk.q_stride : nullptr;
-  const int* __restrict__ bt = bk.block_table + (int64_t)box * bk.bt_stride;
-
-  // ---- round trip 1: everything that depends on the box index only ---------------------
-  const int rank = bk.rank[box];
-  int nseq = bk.num_seqs[box];
-  int kv = bk.kv[box];
-  // this lane's row: sequence id and partial-slot ordinal (the plan's own rank, or - when the
-  // caller supplies it - the box's ordinal among the boxes of that sequence)
+  // this lane's row: sequence id and partial-result slot (-1: no such row)
   const int my_j = (row0 + n) / G;
-  const bool j_ok = my_j < bk.max_seqs;
-  const int my_seq_raw = j_ok ? qt[my_j] : -1;
-  const int my_ord = (j_ok && qs) ? qs[my_j] : rank;
-  // page ids of the chunk: lane i of every wave holds pages i and 64 + i
-  const int first_page = t_begin / page;
-  int pg0 = (first_page + lane < bk.max_blocks) ? bt[first_page + lane] : 0;
-  int pg1 = (first_page + 64 + lane < bk.max_blocks) ? bt[first_page + 64 + lane] : 0;
-  pg0 = pg0 < 0 ? 0 : (pg0 >= p.num_pages ? p.num_pages - 1 : pg0);
-  pg1 = pg1 < 0 ? 0 : (pg1 >= p.num_pages ? p.num_pages - 1 : pg1);
+  const bool j_ok = (row0 + n < R) && my_j < record_max_seqs;
+  const int* __restrict__ rows_tab = (const int*)(rec + sizeof(RecordHead));
+  const int my_seq = j_ok ? rows_tab[my_j] : -1;
+  const int my_sl = j_ok ? rows_tab[record_max_seqs + my_j] : -1;
+  // page ids of the piece: lane i of every wave holds pages i and 64 + i (the record kernel
+  // filled all kMaxChunkPages-or-fewer entries it reserved, so no bound is checked here)
+  const int* __restrict__ pages_tab = rows_tab + 2 * record_max_seqs;
+  const int npages = (ntok + page - 1) / page;
+  const int pg0 = (lane < npages) ? pages_tab[lane] : 0;
+  const int pg1 = (64 + lane < npages) ? pages_tab[64 + lane] : 0;
 
-  nseq = nseq < 0 ? 0 : (nseq > bk.max_seqs ? bk.max_seqs : nseq);
-  int R = nseq * G;
-  const int row_cap = shared_tiles ? 64 : 16;
-  if (R > row_cap) R = row_cap;
-  const int kv_cap = bk.max_blocks * page;
-  kv = kv < 0 ? 0 : (kv > kv_cap ? kv_cap : kv);
-  if (R == 0) return;
   const bool has_rows = row0 < R;   // false: a wave that only helps loading shared tiles
-
-  const bool row_ok = (row0 + n < R) && ((unsigned)my_seq_raw < (unsigned)p.batch) &&
-                      ((unsigned)my_ord < (unsigned)p.max_split);
+  const bool row_ok = my_seq >= 0 && my_sl >= 0;
   const int my_hq = head * G + (row0 + n) % G;
-  // first partial slot of (my row, this box); -1: the row is not to be written
-  const int my_slot0 = row_ok ? (my_seq_raw * p.heads + my_hq) * p.num_slots + my_ord * p.chunks_per_rank : -1;
+  // partial slot of (my row, this piece); -1: the row is not to be written
+  const int my_slot0 = row_ok ? (my_seq * p.heads + my_hq) * p.num_slots + my_sl : -1;
 
   // ---- where a finished row goes ---------------------------------------------------------
   // Normally into its partial slot (fp32, merged by the second kernel). A launch in which every
   // row has exactly one slot (no sequence in two boxes, no box in two chunks) has nothing to
   // merge: its rows go straight to `out` in the output type (the reference does the same when
-  // max_split_per_seq is 1, csrc/api.h:230-238). A row's first slot index is then its
-  // (sequence, head) pair.
+  // max_split_per_seq is 1, csrc/api.h:230-238). A row's slot index is then its (sequence, head)
+  // pair.
   constexpr bool direct = DIRECT;
   auto row_out = [&](int slot0) -> T* {
     const int s_ = slot0 / p.heads;
@@ -200,26 +186,25 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     else if (p.lse_out != nullptr) p.lse_out[prow] = lse;
   };
 
-  // ---- slots of this box that no workgroup will fill are marked empty (-inf) ------------
+  // ---- slots of these rows that no workgroup will fill are marked empty (-inf) -----------
   {
-    const bool empty = t_begin >= kv;
-    const int first = empty ? chunk : chunk + 1;
-    const int last = (chunk == bk.chunks - 1) ? p.chunks_per_rank : chunk + 1;  // exclusive
+    const bool empty = ntok <= 0;
+    const bool marker = (shared_tiles || head_per_wave || wave == 0) && my_slot0 >= 0;
     if (direct) {
-      // (one chunk per box: only a box without tokens gets here; its rows are zero, LSE -inf)
-      if (empty && (shared_tiles || head_per_wave || wave == 0) && my_slot0 >= 0) {
+      // (one piece per box: only a box without tokens gets here; its rows are zero, LSE -inf)
+      if (empty && marker) {
         T* o = row_out(my_slot0) + g * 4;
 #pragma unroll
         for (int db = 0; db < DB; ++db) put4(nullptr, o + db * 16, f32x4{0.f, 0.f, 0.f, 0.f});
         if (g == 0) put_lse(my_slot0, neg_inf());
       }
-    } else if ((shared_tiles || head_per_wave || wave == 0) && g == 0 && my_slot0 >= 0)
-      for (int c = first; c < last; ++c) p.lse_part[my_slot0 + c] = neg_inf();
+    } else if (marker && g == 0)
+      for (int c = fill_begin; c < fill_end; ++c) p.lse_part[my_slot0 + c] = neg_inf();
     if (empty) return;
   }
-  const int t_end = (kv < t_begin + bk.chunk_tokens) ? kv : t_begin + bk.chunk_tokens;
-  const int last_rel = t_end - t_begin - 1;
-  const int nsteps = (t_end - t_begin + kStepTokens - 1) / kStepTokens;
+  const int t_begin = 0, t_end = ntok;   // token positions are piece-relative from here on
+  const int last_rel = ntok - 1;
+  const int nsteps = (ntok + kStepTokens - 1) / kStepTokens;
 
   // ---- addressing ---------------------------------------------------------------------------
   // A 16-token half of a step never straddles a page, so its rows share one base address that is
@@ -231,7 +216,6 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   const int64_t vsp = p.v_stride_page * (int64_t)sizeof(T), vss = p.v_stride_slot * (int64_t)sizeof(T);
   const char* __restrict__ kbase = (const char*)p.k + (int64_t)head * p.k_stride_h * (int64_t)sizeof(T);
   const char* __restrict__ vbase = (const char*)p.v + (int64_t)head * p.v_stride_h * (int64_t)sizeof(T);
-  const int ntok = t_end - t_begin;
 
   // base address of half h (chunk-relative, uniform, h * 16 <= last_rel)
   auto half_base = [&](const char* base, int64_t sp, int64_t ss, int h) -> const char* {
@@ -267,8 +251,8 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
   // Q rows as MFMA B operand (lane (g, n): row row0 + n, dims kk*32 + g*8 .. +7)
   vec8 qreg[KK];
   auto load_q = [&]() {
-    const bool ok = (row0 + n < R) && ((unsigned)my_seq_raw < (unsigned)p.batch);
-    const T* qrow = (const T*)p.q + (ok ? ((int64_t)my_seq_raw * p.q_stride_b + (int64_t)my_hq * p.q_stride_h) : 0);
+    const bool ok = my_seq >= 0;
+    const T* qrow = (const T*)p.q + (ok ? ((int64_t)my_seq * p.q_stride_b + (int64_t)my_hq * p.q_stride_h) : 0);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       u32x4 raw = u32x4{0u, 0u, 0u, 0u};
@@ -369,7 +353,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     // D = 64: one load per step and thread, waves 2 and 3 read the step's second half
     if (NP == 1 && __builtin_amdgcn_readfirstlane(wave >> 1)) next_half();
     auto fetch = [&](int st, u32x4 (&kd)[NP], u32x4 (&vd)[NP]) {
-      if ((st + 1) * kStepTokens <= ntok) {
+      if ((st + 1) * kStepTokens <= ntok_u) {
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
           const unsigned pg = (unsigned)__builtin_amdgcn_readlane(f_page < 64 ? pg0 : pg1, f_page & 63);
@@ -389,13 +373,13 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     };
 #pragma unroll
     for (int s = 0; s < PF; ++s)
-      if (s < nsteps) fetch(s, kst[s], vst[s]);
+      if (s < nsteps_u) fetch(s, kst[s], vst[s]);
     load_q();
-    for (int st0 = 0; st0 < nsteps; st0 += PF) {
+    for (int st0 = 0; st0 < nsteps_u; st0 += PF) {
 #pragma unroll
       for (int s = 0; s < PF; ++s) {
         const int st = st0 + s;
-        if (st >= nsteps) break;
+        if (st >= nsteps_u) break;
         PAT_LDS char* stage = (PAT_LDS char*)smem + (st & 1) * SHARED;
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
@@ -404,7 +388,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
           *(PAT_LDS u32x4*)(stage + tok_in * RSK + col16) = kst[s][i];
           *(PAT_LDS u32x4*)(stage + kStepTokens * RSK + tok_in * RSV + col16) = vst[s][i];
         }
-        if (st + PF < nsteps) fetch(st + PF, kst[s], vst[s]);
+        if (st + PF < nsteps_u) fetch(st + PF, kst[s], vst[s]);
         __syncthreads();
         if (has_rows)
           attend([&](int a, int kk) { return *(const PAT_LDS vec8*)(stage + (a * 16 + n) * RSK + (kk * 32 + g * 8) * 2); },
@@ -413,7 +397,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     }
     l_run = sum_xor32(sum_xor16(l_run));
     if (my_slot0 >= 0) {
-      const int64_t prow = (int64_t)my_slot0 + chunk;
+      const int64_t prow = (int64_t)my_slot0;
       const float inv = 1.f / l_run;
       float* dst = p.o_part + prow * D + g * 4;
       T* o = direct ? row_out(my_slot0) + g * 4 : nullptr;
@@ -493,7 +477,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
     if (head_per_wave) {
       // the wave has seen the whole chunk of its head: its rows go out as they are
       if (my_slot0 >= 0) {
-        const int64_t prow = (int64_t)my_slot0 + chunk;
+        const int64_t prow = (int64_t)my_slot0;
         const float inv = 1.f / l_run;
         float* dst = p.o_part + prow * D + g * 4;
         T* o = direct ? row_out(my_slot0) + g * 4 : nullptr;
@@ -526,7 +510,7 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
         wsum += wgt[w] * s_l[w][crow];
       }
       const float inv = 1.f / wsum;
-      const int64_t prow = (int64_t)cslot0 + chunk;
+      const int64_t prow = (int64_t)cslot0;
       float* dst = p.o_part + prow * D + ccol;
       T* od = direct ? row_out(cslot0) + ccol : nullptr;
 #pragma unroll
@@ -545,17 +529,18 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const Spli
 }
 
 // Host launcher: picks the instance for (element type, head_dim).
+typedef void (*SplitFn)(const char*, int, int, const SplitParams);
 template <bool DIRECT>
-static void (*split_instance(bool bf16, int head_dim))(const SplitParams) {
+static SplitFn split_instance(bool bf16, int head_dim) {
   if (bf16) return head_dim == 64 ? pat_split_kernel<__bf16, 64, DIRECT> : pat_split_kernel<__bf16, 128, DIRECT>;
   return head_dim == 64 ? pat_split_kernel<_Float16, 64, DIRECT> : pat_split_kernel<_Float16, 128, DIRECT>;
 }
 
 hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const SplitParams& params) {
-  void (*fn)(const SplitParams) = params.direct ? split_instance<true>(bf16, head_dim) : split_instance<false>(bf16, head_dim);
+  SplitFn fn = params.direct ? split_instance<true>(bf16, head_dim) : split_instance<false>(bf16, head_dim);
   const unsigned wgs = (unsigned)params.total_items;
   const dim3 grid(wgs < (unsigned)kGridX ? wgs : (unsigned)kGridX, (wgs + kGridX - 1) / kGridX);
-  hipLaunchKernelGGL(fn, grid, dim3(kThreads), 0, stream, params);
+  hipLaunchKernelGGL(fn, grid, dim3(kThreads), 0, stream, params.records, params.record_stride, params.record_max_seqs, params);
   return hipGetLastError();
 }
 

@@ -72,6 +72,8 @@ struct Prepared {
   pat_fwd_args args;
   std::vector<pat_fwd_bucket> buckets;
   TensorList keep;          // plan tensors (and derived slots) stay alive as long as the launch does
+  at::Tensor records;       // the plan's launch records (shared by every launch of the plan)
+  int64_t plan_version = -1;   // version of the plan tables the records were built from
   size_t need = 0;          // workspace bytes
   pat_fwd_tuning tuning;    // the measured geometry of this plan shape (args.tuning points here when set)
   Prepared() { std::memset(&args, 0, sizeof(args)); std::memset(&tuning, 0, sizeof(tuning)); }
@@ -144,6 +146,42 @@ void tune(Prepared& L, const c10::Device& dev) {
   g_tuned[key] = best;
 }
 
+// ---- launch records, shared by the launches of one plan -----------------------------------------
+// The records depend on the plan tables and the launch geometry, not on q / k / v / out: the layers
+// of a model (one prepared launch each) share one set. `version` counts in-place edits of the plan
+// tables (torch's version counter): records of an older version are dropped.
+struct RecordStore {
+  int64_t version = -1;
+  std::unordered_map<uint64_t, at::Tensor> by_tag;
+  // plans that came without slot tables: the ordinals derived on the device (pat_fwd_derive_slots)
+  at::Tensor derived_slots;
+  std::vector<int64_t> derived_offsets;
+  int64_t derived_version = -1;
+};
+
+void attach_records(Prepared& L, RecordStore& store, int64_t version, const c10::Device& dev) {
+  if (store.version != version) { store.by_tag.clear(); store.version = version; }
+  pat_fwd_args& a = L.args;
+  a.records = nullptr;
+  uint64_t tag = 0;
+  check(pat_fwd_records_tag(&a, &tag));
+  auto it = store.by_tag.find(tag);
+  if (it == store.by_tag.end()) {
+    size_t rbytes = 0;
+    check(pat_fwd_records_bytes(&a, &rbytes));
+    at::Tensor records = at::empty({(int64_t)rbytes}, at::TensorOptions().dtype(at::kByte).device(dev));
+    uint64_t built = 0;
+    check(pat_fwd_build_records(&a, records.data_ptr(), rbytes, &built, raw_stream(dev)));
+    if (store.by_tag.size() >= 16) store.by_tag.clear();
+    it = store.by_tag.emplace(built, records).first;
+    tag = built;
+  }
+  L.records = it->second;
+  L.plan_version = version;
+  a.records = L.records.data_ptr(); a.records_bytes = (size_t)L.records.numel(); a.records_tag = tag;
+  check(pat_fwd_workspace_bytes(&a, &L.need));
+}
+
 void strides3(const at::Tensor& t, int64_t out[3]) {
   out[0] = t.stride(0); out[1] = t.stride(1); out[2] = t.stride(2);
 }
@@ -163,7 +201,7 @@ struct PlanTables {
 std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
                                   const at::Tensor& num_split, const PlanTables& pt, int max_split, int max_seqs,
                                   int max_blocks, double scale, const at::Tensor& out,
-                                  const std::optional<at::Tensor>& lse) {
+                                  const std::optional<at::Tensor>& lse, RecordStore& store, int64_t plan_version) {
   require(q.scalar_type() == at::kHalf || q.scalar_type() == at::kBFloat16, "only support fp16 and bf16 data type");
   require(k.scalar_type() == q.scalar_type(), "query and key must have the same dtype");
   require(v.scalar_type() == q.scalar_type(), "query and value must have the same dtype");
@@ -249,18 +287,21 @@ std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, cons
     // A plan without slot tables (the reference's call form): CTA_rank is not unique per sequence on
     // irregular forests, so the ordinals are derived from the q_tables on the device, once per
     // prepared launch (the caches key on the tables' version counters).
-    size_t sbytes = 0;
-    check(pat_fwd_slots_bytes(&a, &sbytes));
-    at::Tensor derived = at::empty({(int64_t)sbytes}, at::TensorOptions().dtype(at::kByte).device(q.device()));
-    std::vector<int64_t> offsets(std::max<size_t>(nb, 1), 0);
-    check(pat_fwd_derive_slots(&a, derived.data_ptr(), sbytes, offsets.data(), raw_stream(q.device())));
-    int32_t* base = static_cast<int32_t*>(derived.data_ptr());
-    for (size_t i = 0; i < nb; ++i) L->buckets[i].q_slot = base + offsets[i];
+    if (!store.derived_slots.defined() || store.derived_version != plan_version) {
+      size_t sbytes = 0;
+      check(pat_fwd_slots_bytes(&a, &sbytes));
+      store.derived_slots = at::empty({(int64_t)sbytes}, at::TensorOptions().dtype(at::kByte).device(q.device()));
+      store.derived_offsets.assign(std::max<size_t>(nb, 1), 0);
+      check(pat_fwd_derive_slots(&a, store.derived_slots.data_ptr(), sbytes, store.derived_offsets.data(), raw_stream(q.device())));
+      store.derived_version = plan_version;
+    }
+    int32_t* base = static_cast<int32_t*>(store.derived_slots.data_ptr());
+    for (size_t i = 0; i < nb; ++i) L->buckets[i].q_slot = base + store.derived_offsets[i];
     a.num_split_per_seq = base;
-    L->keep.push_back(derived);
+    L->keep.push_back(store.derived_slots);
   }
   tune(*L, q.device());
-  check(pat_fwd_workspace_bytes(&a, &L->need));
+  attach_records(*L, store, plan_version, q.device());
   return L;
 }
 
@@ -310,6 +351,17 @@ struct KernelInfo {
   std::optional<at::Tensor> flat;
   pat_flat_plan layout;
   std::unordered_map<std::string, std::shared_ptr<Prepared>> cache;
+  RecordStore records;
+
+  // Counts in-place edits of the plan tables: every table is a view of one buffer, whose version
+  // counter torch advances with each of them (a plan held table by table: the counters' sum).
+  int64_t plan_version() const {
+    if (flat.has_value()) return (int64_t)flat->_version();
+    int64_t v = (int64_t)num_split_per_seq._version() + (int64_t)num_boxes_per_seq._version();
+    for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables})
+      for (const at::Tensor& t : *l) v += (int64_t)t._version();
+    return v;
+  }
 
   void clear_tables() {
     for (TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables, &l_q_tables,
@@ -317,6 +369,7 @@ struct KernelInfo {
       l->clear();
     mnws.clear(); l_mnws.clear(); l_flags.clear(); launch_parts.clear();
     cache.clear();
+    records = RecordStore();
   }
 
   // (Re)creates every plan tensor as a view of `buf` (the host buffer or its copy on a device).
@@ -367,6 +420,7 @@ struct KernelInfo {
     num_split_per_seq = num_split_per_seq.to(device, true);
     num_boxes_per_seq = num_boxes_per_seq.to(device, true);
     cache.clear();
+    records = RecordStore();
   }
 
   py::dict launch_tables() const {
@@ -511,6 +565,7 @@ struct PrefixTreeCPP {
 // ---- forward ------------------------------------------------------------------------------------------
 std::mutex g_table_mutex;
 std::unordered_map<std::string, std::shared_ptr<Prepared>> g_table_launches;
+std::unordered_map<std::string, std::shared_ptr<RecordStore>> g_table_records;   // per plan (tables + versions)
 
 struct DeviceScope {   // the kernels launch on the current HIP device: switch only when q lives elsewhere
   std::optional<c10::DeviceGuard> guard;
@@ -533,19 +588,22 @@ void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, c
   // The prepared launch is kept per set of tensors: a decode step calls this once per layer with the
   // same plan. The key holds what the argument block was built from (addresses, layouts, version
   // counters of the plan tensors); the tensors' contents are read by the kernels at every call.
+  Key plan_key;
+  plan_key.plan_tensor(num_split);
+  for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs}) {
+    plan_key.add((int64_t)l->size());
+    for (const at::Tensor& t : *l) plan_key.plan_tensor(t);
+  }
+  for (const auto& m : mnw) for (int x : m) plan_key.add(x);
+  plan_key.add(max_split); plan_key.add(max_seqs); plan_key.add(max_blocks);
+  plan_key.add(slot_tables.has_value());
+  if (slot_tables.has_value()) for (const at::Tensor& t : *slot_tables) plan_key.plan_tensor(t);
+  if (bucket_flags.has_value()) for (int f : *bucket_flags) plan_key.add(f);
   Key key;
   key.tensor(q); key.tensor(k); key.tensor(v); key.tensor(out);
   key.add(lse.has_value()); if (lse.has_value()) key.tensor(*lse);
-  key.plan_tensor(num_split);
-  for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs}) {
-    key.add((int64_t)l->size());
-    for (const at::Tensor& t : *l) key.plan_tensor(t);
-  }
-  for (const auto& m : mnw) for (int x : m) key.add(x);
-  key.add(max_split); key.add(max_seqs); key.add(max_blocks); key.add(scale);
-  key.add(slot_tables.has_value());
-  if (slot_tables.has_value()) for (const at::Tensor& t : *slot_tables) key.plan_tensor(t);
-  if (bucket_flags.has_value()) for (int f : *bucket_flags) key.add(f);
+  key.add(scale);
+  key.bytes += plan_key.bytes;
 
   std::shared_ptr<Prepared> L;
   {
@@ -557,7 +615,16 @@ void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, c
     PlanTables pt{&q_tables, &block_tables, &num_seqs, &ranks, &kvs,
                   slot_tables.has_value() ? &*slot_tables : nullptr, &mnw,
                   bucket_flags.has_value() ? &*bucket_flags : nullptr};
-    L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse);
+    // the launch records belong to the plan (tables + their versions), not to q / k / v / out
+    std::shared_ptr<RecordStore> store;
+    {
+      std::lock_guard<std::mutex> lock(g_table_mutex);
+      if (g_table_records.size() >= 16) g_table_records.clear();
+      auto& slot = g_table_records[plan_key.bytes];
+      if (!slot) slot = std::make_shared<RecordStore>();
+      store = slot;
+    }
+    L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse, *store, 0);
     std::lock_guard<std::mutex> lock(g_table_mutex);
     if (g_table_launches.size() >= 64) g_table_launches.clear();
     g_table_launches[key.bytes] = L;
@@ -575,9 +642,12 @@ void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, Pre
   key.tensor(q); key.tensor(k); key.tensor(v); key.tensor(out); key.add(scale);
   key.add(lse.has_value()); if (lse.has_value()) key.tensor(*lse);
   std::shared_ptr<Prepared> L;
+  const int64_t version = info.plan_version();
   auto it = info.cache.find(key.bytes);
   if (it != info.cache.end()) {
     L = it->second;
+    // the plan tables were edited in place since (DecodePlan.advance_step): records of the new contents
+    if (L->plan_version != version) attach_records(*L, info.records, version, q.device());
   } else {
     const bool l = info.has_launch;
     const std::vector<int> no_flags;
@@ -588,7 +658,8 @@ void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, Pre
                   l ? &info.l_slot_tables : &info.slot_tables, l ? &info.l_mnws : &info.mnws,
                   l ? &info.l_flags : &no_flags};
     require(!pt.mnw->empty(), "the tree has no plan: call pack_schedule and kernel_info.to_gpu first");
-    L = prepare(q, k, v, info.num_boxes_per_seq, pt, info.max_boxes, info.max_seqs, info.max_blocks, scale, out, lse);
+    L = prepare(q, k, v, info.num_boxes_per_seq, pt, info.max_boxes, info.max_seqs, info.max_blocks, scale, out, lse,
+                info.records, version);
     if (info.cache.size() >= 256) info.cache.clear();
     info.cache[key.bytes] = L;
   }

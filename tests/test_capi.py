@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"libpat_amd.so does not export {name}"
     assert sorted(_lib.SYMBOLS) == names       # the ctypes table covers the header, no more, no less
-    assert lib.pat_abi_version() == 2
+    assert lib.pat_abi_version() == 3
 
 
 def _args(**over):
@@ -127,7 +127,8 @@ def test_geometry_and_workspace_are_consistent():
 
 def test_single_slot_launch_needs_no_workspace(tuning):
     # no sequence in two boxes (max_split_per_seq 1), every box one chunk, a box per CU and kv head:
-    # the launch writes `out` from its first kernel (csrc/api.h:230-238) and needs no scratch
+    # the launch writes `out` from its first kernel (csrc/api.h:230-238) and, given the plan's
+    # launch records, needs no scratch
     lib = _lib.load()
     fake = 0x10000
 
@@ -138,7 +139,7 @@ def test_single_slot_launch_needs_no_workspace(tuning):
         b[0].num_boxes, b[0].max_seqs, b[0].max_blocks = boxes, 1, blocks
         b[0].mnw[0], b[0].mnw[1], b[0].mnw[2] = 16, 128, 1
         kw = dict(batch=boxes, max_split_per_seq=1, max_seqs_in_box=1, max_blocks_in_box=blocks, num_buckets=1,
-                  buckets=C.cast(b, C.POINTER(_lib.FwdBucket)))
+                  buckets=C.cast(b, C.POINTER(_lib.FwdBucket)), records=fake)
         kw.update(over)
         a = _args(**kw)
         a._keep = b
@@ -161,6 +162,38 @@ def test_single_slot_launch_needs_no_workspace(tuning):
     tuning(direct_out=0)
     g, need = plan(64, 100)
     assert g.num_slots == 1 and need > 0
+    # without prebuilt records the launch writes them into its workspace: one per workgroup
+    tuning()
+    g, need = plan(64, 100, records=0)
+    rec = C.c_size_t()
+    a = _args()
+    assert need > 0 and need % 256 == 0 and need >= g.num_workgroups * 64
+
+
+def test_record_buffer_sizes_and_errors_without_a_gpu():
+    lib = _lib.load()
+    a = _args()
+    g, need, rec = _lib.FwdGeometry(), C.c_size_t(), C.c_size_t()
+    assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
+    assert lib.pat_fwd_records_bytes(C.byref(a), C.byref(rec)) == 0
+    # a record: 32-byte header, sequence id and slot per sequence of the widest box (16), page ids of the
+    # longest piece, rounded up to 64 bytes
+    pages = max(g.chunk_tokens, g.tall_chunk_tokens) // 16
+    assert rec.value >= g.num_workgroups * (32 + 2 * 16 * 4 + 4)
+    assert rec.value <= 256 + g.num_workgroups * ((32 + 2 * 16 * 4 + pages * 4 + 63) // 64 * 64)
+    # the launch's own workspace holds the partial results and, without prebuilt records, the records
+    assert lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)) == 0
+    with_records = C.c_size_t()
+    b = _args(records=0x20000)
+    assert lib.pat_fwd_workspace_bytes(C.byref(b), C.byref(with_records)) == 0
+    assert need.value == with_records.value + rec.value
+    tag = C.c_uint64()
+    assert lib.pat_fwd_build_records(C.byref(a), None, 0, C.byref(tag), None) == _lib.PAT_ERR_INVALID
+    assert lib.pat_fwd_build_records(C.byref(a), C.c_void_p(0x10000), 16, C.byref(tag), None) == _lib.PAT_ERR_WORKSPACE
+    assert lib.pat_fwd_build_records(C.byref(a), C.c_void_p(0x10010), rec.value, C.byref(tag), None) == _lib.PAT_ERR_WORKSPACE
+    # records whose tag does not belong to this launch are refused before any GPU call
+    b.workspace, b.workspace_bytes, b.records_bytes, b.records_tag = 0x100000, with_records.value, rec.value, 12345
+    assert lib.pat_fwd_launch(C.byref(b), None) == _lib.PAT_ERR_INVALID and "launch records" in _lib.last_error()
 
 
 def test_static_scratch_and_slot_buffer_sizes_without_a_gpu():
