@@ -17,8 +17,13 @@
 
 namespace pat {
 
+// (the leading scalar arguments repeat the fields of `p` that the first two memory reads need:
+// they are preloaded into SGPRs with the wave, the rest of `p` arrives by load meanwhile)
 template <typename T, int D>
-__global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
+__global__ void __launch_bounds__(256) pat_merge_kernel(const int32_t* __restrict__ num_split_per_seq,
+                                                        const float* __restrict__ lse_part, const int num_slots,
+                                                        const int chunks_per_rank, const int max_split, const int batch,
+                                                        const int heads, const int kv_heads, const MergeParams p) {
   constexpr int CPL = D / 64;   // columns per lane
   constexpr int kRegs = 4;      // LSE registers per lane: up to 256 slots stay in registers
   constexpr int kBatch = 16;    // partial rows fetched together
@@ -28,29 +33,29 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const MergeParams p) {
   // (where most of it still sits): with a multiple of 8 kv heads, workgroup b serves heads of the kv
   // heads = b mod 8, so the rows are found in its own L2. A matter of speed only.
   int s, hq;
-  if (p.kv_heads % 8 == 0) {
+  if (kv_heads % 8 == 0) {
     const int xcd = blockIdx.x & 7;
-    const int per_seq = p.heads >> 3;                       // heads of one sequence served by one XCD
+    const int per_seq = heads >> 3;                       // heads of one sequence served by one XCD
     const int64_t u = (int64_t)(blockIdx.x >> 3) * 4 + (threadIdx.x >> 6);
-    if (u >= (int64_t)p.batch * per_seq) return;
+    if (u >= (int64_t)batch * per_seq) return;
     s = (int)(u / per_seq);
     const int local = (int)(u - (int64_t)s * per_seq);      // kv head (xcd + 8 i), head g of its group
-    const int group = p.heads / p.kv_heads;
+    const int group = heads / kv_heads;
     hq = (xcd + 8 * (local / group)) * group + local % group;
   } else {
     const int64_t u = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (u >= (int64_t)p.batch * p.heads) return;
-    s = (int)(u / p.heads);
-    hq = (int)(u % p.heads);
+    if (u >= (int64_t)batch * heads) return;
+    s = (int)(u / heads);
+    hq = (int)(u % heads);
   }
-  const int64_t pair = (int64_t)s * p.heads + hq;
+  const int64_t pair = (int64_t)s * heads + hq;
   const float ninf = -__builtin_inff();
 
-  const float* __restrict__ lse = p.lse_part + pair * p.num_slots;
-  const float* __restrict__ op = p.o_part + pair * (int64_t)p.num_slots * D;
-  int nsplit = p.num_split_per_seq[s];
-  nsplit = nsplit < 0 ? 0 : (nsplit > p.max_split ? p.max_split : nsplit);
-  const int nslots = nsplit * p.chunks_per_rank;  // slots are box-major
+  const float* __restrict__ lse = lse_part + pair * num_slots;
+  const float* __restrict__ op = p.o_part + pair * (int64_t)num_slots * D;
+  int nsplit = num_split_per_seq[s];
+  nsplit = nsplit < 0 ? 0 : (nsplit > max_split ? max_split : nsplit);
+  const int nslots = nsplit * chunks_per_rank;  // slots are box-major
 
   // slot LSEs -> registers (slots past 256 are re-read below; no plan of the default buckets
   // gets there: 32 splits x 64 chunks would)
@@ -136,10 +141,11 @@ hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const Merge
   // (a multiple of 8 kv heads: 8 interleaved lists of pairs, one per XCD, each rounded up to whole workgroups)
   const int64_t wgs = params.kv_heads % 8 == 0 ? 8 * ((pairs / 8 + 3) / 4) : (pairs + 3) / 4;
   const dim3 grid((unsigned)wgs), block(256);
-  void (*fn)(const MergeParams);
+  void (*fn)(const int32_t*, const float*, int, int, int, int, int, int, const MergeParams);
   if (bf16) fn = head_dim == 64 ? pat_merge_kernel<__bf16, 64> : pat_merge_kernel<__bf16, 128>;
   else fn = head_dim == 64 ? pat_merge_kernel<_Float16, 64> : pat_merge_kernel<_Float16, 128>;
-  hipLaunchKernelGGL(fn, grid, block, 0, stream, params);
+  hipLaunchKernelGGL(fn, grid, block, 0, stream, params.num_split_per_seq, params.lse_part, params.num_slots,
+                     params.chunks_per_rank, params.max_split, params.batch, params.heads, params.kv_heads, params);
   return hipGetLastError();
 }
 

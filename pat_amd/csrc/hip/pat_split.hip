@@ -82,7 +82,8 @@ __global__ void __launch_bounds__(kThreads, PAT_OCC) pat_split_kernel(const char
   constexpr int DB = D / 16;             // 16-wide head_dim blocks of O^T
   constexpr int NV = D / 16;             // 16-byte V loads per lane per step (wave-private tiles)
   constexpr int NP = D / 64;             // 16-byte K (and V) loads per thread per step (shared tiles)
-  constexpr int PF = 4;                  // shared tiles: steps kept in flight per workgroup
+  constexpr int PF = 3;                  // shared tiles: steps kept in flight per workgroup (a 4th costs the 16 registers that let the
+                                         // operand reads of a step run ahead of its MFMAs: lone tall workgroups 6 % slower per step)
   constexpr int DEPTH = PAT_DEPTH;       // wave-private tiles: steps kept in flight per wave
   constexpr int CPR = D / 8;             // 16-byte pieces per token row
   constexpr int TPL = 64 / CPR;          // tokens covered by one wave-wide load instruction

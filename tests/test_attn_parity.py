@@ -774,3 +774,61 @@ def test_autotuned_geometry_matches_oracle_and_is_remembered():
         assert len(chosen) == 2 and chosen[0] == chosen[1] and len(chosen[0]) == 7
     finally:
         _prefix_attn.set_autotune(was)
+
+
+@pytest.mark.parametrize("name", ["c2", "c4"])
+def test_launch_records_prebuilt_or_built_by_the_launch(name):
+    # The launch records of a plan (one per workgroup: rows, slots, pages) built once with
+    # pat_fwd_build_records and handed to the launch, against a launch that builds them itself in its
+    # workspace, against pat_fwd_launch_static doing the same in the built-in scratch: identical bits,
+    # and the oracle's values. Records of another geometry are refused.
+    print(f"[case] launch records, {name}: prebuilt / built by the launch / built in the static scratch", flush=True)
+    import ctypes as C
+    from pat_amd import _ctypes_launch, _lib
+    lib = _lib.load()
+    dev = _device()
+    w = workloads.make(name, seed=0)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    lt = info.launch_tables()
+    stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    results = []
+    for route in ("prebuilt", "by the launch", "static scratch"):
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+        L = _ctypes_launch.prepare(q, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
+                                   lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
+                                   info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                                   1.0 / math.sqrt(w.head_dim), out, lse, lt["slot_tables"], lt.get("flags"),
+                                   build_records=route == "prebuilt")
+        assert (L.args.records is not None) == (route == "prebuilt")
+        if route == "static scratch":
+            assert L.need <= lib.pat_fwd_static_scratch_bytes()
+            L.args.workspace, L.args.workspace_bytes = None, 0
+            rc = lib.pat_fwd_launch_static(C.byref(L.args), stream)
+        else:
+            ws = torch.empty(L.need, dtype=torch.uint8, device=dev)
+            L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), L.need
+            rc = lib.pat_fwd_launch(C.byref(L.args), stream)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        results.append((route, L, out, lse))
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"{name} prebuilt records", results[0][2], results[0][3], ref_out, ref_lse, w.dtype)
+    for route, _, out, lse in results[1:]:
+        assert torch.equal(out, results[0][2]) and torch.equal(lse, results[0][3]), route
+    # the workspace of a launch that builds its own records is larger by exactly the records
+    rbytes = C.c_size_t()
+    assert lib.pat_fwd_records_bytes(C.byref(results[1][1].args), C.byref(rbytes)) == 0
+    assert results[1][1].need == results[0][1].need + rbytes.value
+    # records that belong to another geometry: refused, nothing enqueued
+    L = results[0][1]
+    L.args.records_tag ^= 1
+    ws = torch.empty(max(L.need, 256), dtype=torch.uint8, device=dev)
+    L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), L.need
+    assert lib.pat_fwd_launch(C.byref(L.args), stream) == _lib.PAT_ERR_INVALID
+    assert "launch records" in _lib.last_error()
