@@ -3,6 +3,10 @@
 Public API = the `prefix_attn` API of flashserve/PAT (prefix_attn/__init__.py:10-26),
 implemented over libpat_amd (C ABI in include/pat_amd.h; HIP kernels for gfx950).
 """
+# torch first: its libraries (and the HIP runtime under them) must be initialised before, and torn down
+# after, the extension and libpat_amd that use them - loaded the other way round, the process ends
+# in a crash inside the heap's clean-up when it exits
+import torch  # noqa: F401
 try:
     from ._prefix_attn import prefix_attn_with_kvcache, PrefixTreeCPP, paged_decode_baseline
 except ImportError as exc:   # no fallback: the compiled binding and libpat_amd.so are the product

@@ -126,8 +126,10 @@ void tune(Prepared& L, const c10::Device& dev) {
   L.args.workspace = ws.data_ptr(); L.args.workspace_bytes = (size_t)ws.numel();
   // 320 MB per device, read between the timed launches (more than the 256 MB memory-side cache holds):
   // allocated at the first measurement and kept
+  // (held for the life of the process and never destroyed: a static destructor would release device
+  // memory after the HIP runtime has shut down)
   static std::mutex evict_mutex;
-  static std::unordered_map<int, at::Tensor> evict_buffers;
+  static auto& evict_buffers = *new std::unordered_map<int, at::Tensor>();
   at::Tensor evict;
   {
     std::lock_guard<std::mutex> lock(evict_mutex);
@@ -564,8 +566,9 @@ struct PrefixTreeCPP {
 
 // ---- forward ------------------------------------------------------------------------------------------
 std::mutex g_table_mutex;
-std::unordered_map<std::string, std::shared_ptr<Prepared>> g_table_launches;
-std::unordered_map<std::string, std::shared_ptr<RecordStore>> g_table_records;   // per plan (tables + versions)
+// (both hold device tensors and live until the process ends, undestroyed: see the evict buffers)
+auto& g_table_launches = *new std::unordered_map<std::string, std::shared_ptr<Prepared>>();
+auto& g_table_records = *new std::unordered_map<std::string, std::shared_ptr<RecordStore>>();   // per plan (tables + versions)
 
 struct DeviceScope {   // the kernels launch on the current HIP device: switch only when q lives elsewhere
   std::optional<c10::DeviceGuard> guard;

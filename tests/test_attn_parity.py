@@ -832,3 +832,20 @@ def test_launch_records_prebuilt_or_built_by_the_launch(name):
     L.args.workspace, L.args.workspace_bytes = ws.data_ptr(), L.need
     assert lib.pat_fwd_launch(C.byref(L.args), stream) == _lib.PAT_ERR_INVALID
     assert "launch records" in _lib.last_error()
+
+
+def test_process_that_imports_the_package_first_exits_cleanly():
+    # `python -m pat_amd.bench_trees` imports the package before anything imported torch; the package
+    # must bring torch (and the HIP runtime) up first, or the process crashes in the heap's clean-up
+    # when it exits (after printing correct results). One small tree, in a child process.
+    print("[case] python -m pat_amd.bench_trees in a child process: exit status", flush=True)
+    import os
+    import subprocess
+    import sys
+    _device()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-m", "pat_amd.bench_trees", "--trees", "1,256_256,32", "--heads", "32 8",
+                          "--iters", "2", "--warmup", "1"], cwd=root, capture_output=True, text=True, timeout=110)
+    print(res.stdout[-300:], flush=True)
+    assert res.returncode == 0, f"exit status {res.returncode}: {res.stderr[-500:]}"
+    assert "1,256_256,32" in res.stdout
