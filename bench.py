@@ -35,24 +35,25 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 INFINITY_CACHE_BYTES = 256 << 20
 
 
-def measured_traffic_bytes(workload: str, seed: int):
+def measured_traffic_bytes(workload: str, seed: int, workgroups: int):
     """HBM bytes per split-kernel launch as rocprofv3 measured them (--pmc FETCH_SIZE + WRITE_SIZE, each
-    scaled by the same counter's reading for a 1 GiB copy kernel), from the marker line of
-    profiles/pat_split_kernel_<workload>.md. None when there is no such measurement for this
-    workload and seed, or when the kernel sources have changed since it was taken."""
+    scaled by the same counter's reading for a 1 GiB copy kernel), from the marker lines of
+    profiles/pat_split_kernel_<workload>.md (one per launch geometry that was measured). None when
+    there is no such measurement for this workload, seed and number of workgroups, or when the
+    kernel sources have changed since it was taken."""
     import hashlib
     import re
     path = os.path.join(ROOT, "profiles", f"pat_split_kernel_{workload}.md")
     if not os.path.exists(path):
         return None
-    m = re.search(r"bench-marker: workload=(\S+) seed=(\d+) traffic_bytes=(\d+) kernel_sources_sha256=([0-9a-f]+)",
-                  open(path).read())
-    if m is None or m.group(1) != workload or int(m.group(2)) != seed:
-        return None
     h = hashlib.sha256()
     for rel in ("pat_amd/csrc/hip/pat_split.hip", "pat_amd/csrc/hip/fwd_params.hpp", "pat_amd/csrc/capi_fwd.hip"):
         h.update(open(os.path.join(ROOT, rel), "rb").read())
-    return int(m.group(3)) if h.hexdigest() == m.group(4) else None
+    for m in re.finditer(r"bench-marker: workload=(\S+) seed=(\d+) workgroups=(\d+) traffic_bytes=(\d+) "
+                         r"kernel_sources_sha256=([0-9a-f]+)", open(path).read()):
+        if m.group(1) == workload and int(m.group(2)) == seed and int(m.group(3)) == workgroups and h.hexdigest() == m.group(5):
+            return int(m.group(4))
+    return None
 
 WORKLOAD_TEXT = {
     "c1": "8 req, 256 shared + 32 private tokens, 8/8 heads, d64, fp16",
@@ -242,7 +243,7 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
                      "traffic": None},
     }
 
-    result["roofline"]["traffic"] = measured_traffic_bytes(workload, a.seed)
+    result["roofline"]["traffic"] = measured_traffic_bytes(workload, a.seed, int(geo.num_workgroups))
 
     # the same steps through the drop-in call of the compiled extension (tree form): argument checks
     # and launch preparation are cached per (q, k, v, out), the workspace comes from torch's
