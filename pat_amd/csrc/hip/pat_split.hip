@@ -12,7 +12,8 @@
 //  * work item = (box, kv-head, KV chunk), one workgroup of 4 wave64 each, launched as a flat
 //    list with the kv-head fastest: workgroups are dealt to the 8 XCDs round-robin, so with 8
 //    kv-heads XCD x serves head x and boxes that share KV pages (the boxes of one prefix node)
-//    find them in that XCD's L2. Inside a bucket the list is chunk-major (see the decode below).
+//    find them in that XCD's L2. Inside a bucket the list is chunk-major. What a workgroup is to do
+//    it reads from its launch record (fwd_params.hpp), written once per plan by the record kernel.
 //  * buckets of very short boxes: one workgroup serves 4 kv heads, one per wave, each wave
 //    walking its head's steps alone (no combine).
 //  * boxes of up to 16 rows (one MFMA row tile): each wave owns every 4th 32-token step of
@@ -28,8 +29,8 @@
 //    in padded LDS rows and are read back transposed with ds_read_b64_tr_b16.
 //  * all softmax state of a row lives in the 4 lanes {n, n+16, n+32, n+48}.
 //  * the chunk's page ids live in two VGPRs per wave (lane i holds page i) and are
-//    broadcast with v_readlane, so the prologue is two dependent memory round trips:
-//    {plan scalars, page ids, sequence ids} -> {K, V, Q}.
+//    broadcast with v_readlane; with the launch record the prologue is two dependent memory
+//    round trips: {record: header, sequence ids, slots, page ids} -> {K, V, Q}.
 #include <hip/hip_runtime.h>
 
 #include "fwd_params.hpp"
