@@ -337,7 +337,10 @@ int pat_fwd_build_records(const pat_fwd_args* args, void* buffer, size_t buffer_
 /* prefix_attn_with_kvcache(...)   csrc/bindings.cpp:7-72 -> csrc/api.h:110-295
  * Enqueues the split-KV kernel and (unless the workspace size is 0, see above) the merge
  * kernel on `hip_stream` (a hipStream_t; NULL = the null stream) of the current device and
- * returns without synchronising. */
+ * returns without synchronising. Rows of `out` (and `lse_out`) whose sequence sits in no box of
+ * the plan: the merge kernel writes 0 (LSE -inf) there; a single-slot launch, which has no merge
+ * kernel, leaves them as they were (the scheduler's plans put every sequence in a box; only a
+ * hand-made plan can leave one out). */
 int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
 
 /* pat_fwd_launch for callers that cannot allocate device memory (code under HIP graph capture,
