@@ -355,9 +355,19 @@ def test_manual_fixture_partial_pages():
 
 @pytest.mark.parametrize("spec,heads", [("1,4,16_32,256,32", (64, 8)), ("1,8_640,32", (64, 8)),
                                         ("1,2,4,8,16,32,64_32,512,32,256,32,32,32", (64, 8)),
-                                        ("4,16_4096,256", (32, 32)), ("1,10_4096,416", (16, 8))])
+                                        ("4,16_4096,256", (32, 32)), ("1,10_4096,416", (16, 8)),
+                                        # the rest of the reference's list, at its own 64/8 heads
+                                        ("1,2,4,16,32,64,128,256,512_3072,1024,32,32,32,32,32,32,32", (64, 8)),
+                                        ("1,2,4,16,32,64,256_4096,32,128,128,32,256,512", (64, 8)),
+                                        ("1,2,4,16,32,64,128,256,512_3072,1024,512,256,128,32,256,512,32", (64, 8)),
+                                        ("1,2,4,16,32,64,128,256,1024_512,32,128,128,32,256,512,32,32", (64, 8)),
+                                        ("1,2,4,16,32,64,128,512_512,32,128,128,32,256,512,256", (64, 8)),
+                                        ("1,2,4,16,32,64,128_512,32,128,128,32,256,512", (64, 8)),
+                                        ("4_4096", (64, 8)), ("1,4,256_32,256,32", (64, 8)),
+                                        ("1,16,32_2048,1024,256", (64, 8)), ("4,16_4096,256", (64, 8)),
+                                        ("1,10_4096,416", (64, 8))])
 def test_reference_tree_specs_page32(spec, heads):
-    # tree batches of the reference's own test (test/test.py:174-187): page 32, fp16, d 128
+    # tree batches of the reference's own test (test/test.py:174-187, all 14 of them): page 32, fp16, d 128
     print(f"[case] tree spec {spec} heads {heads}", flush=True)
     import random
     from pat_amd import generate_tree_seqs
