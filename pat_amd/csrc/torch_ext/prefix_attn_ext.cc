@@ -159,6 +159,9 @@ struct RecordStore {
   at::Tensor derived_slots;
   std::vector<int64_t> derived_offsets;
   int64_t derived_version = -1;
+  // a store looked up by the plan tensors' addresses holds those tensors: as long as it exists no
+  // other plan can be allocated at the same addresses and find records that are not its own
+  TensorList keep;
 };
 
 void attach_records(Prepared& L, RecordStore& store, int64_t version, const c10::Device& dev) {
@@ -624,7 +627,13 @@ void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, c
       std::lock_guard<std::mutex> lock(g_table_mutex);
       if (g_table_records.size() >= 16) g_table_records.clear();
       auto& slot = g_table_records[plan_key.bytes];
-      if (!slot) slot = std::make_shared<RecordStore>();
+      if (!slot) {
+        slot = std::make_shared<RecordStore>();
+        slot->keep.push_back(num_split);
+        for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs})
+          for (const at::Tensor& t : *l) slot->keep.push_back(t);
+        if (slot_tables.has_value()) for (const at::Tensor& t : *slot_tables) slot->keep.push_back(t);
+      }
       store = slot;
     }
     L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse, *store, 0);

@@ -859,3 +859,50 @@ def test_process_that_imports_the_package_first_exits_cleanly():
     print(res.stdout[-300:], flush=True)
     assert res.returncode == 0, f"exit status {res.returncode}: {res.stderr[-500:]}"
     assert "1,256_256,32" in res.stdout
+
+
+def test_table_form_new_plan_at_recycled_addresses():
+    # A serving loop drops a plan and builds the next one: same shapes, other contents, and the
+    # allocator hands out the addresses just freed. What the binding remembers per plan (launch
+    # records, derived slots) is looked up by address, so it must not outlive the plan's tensors.
+    print("[case] table form, a new plan at the addresses of a dropped one", flush=True)
+    dev = _device()
+
+    def plan(w):
+        t = PrefixTree(w.page_size)
+        t.build_radix_tree(w.seq_lens, w.rows)
+        ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+        ki.to_tensor(device=dev)
+        return ki
+
+    def call(w, ki, q, k, v, out):
+        prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                                 ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                                 ki.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), out, None)
+
+    wa, wb = workloads.make("c1", seed=0), workloads.make("c1", seed=1)
+    assert wa.rows != wb.rows and [len(r) for r in wa.rows] == [len(r) for r in wb.rows]
+    qa, ka, va = wa.tensors(dev)
+    ki = plan(wa)
+    addresses = [t.data_ptr() for t in ki.block_tables]
+    out = torch.full_like(qa, float("nan"))
+    call(wa, ki, qa, ka, va, out)
+    # more launches of another plan than the binding remembers: the first plan's launch is forgotten
+    wc = _ragged_forest_workload(3, (8, 4), 64, torch.float16)
+    qc, kc, vc = wc.tensors(dev)
+    kic = plan(wc)
+    outs = [torch.empty_like(qc) for _ in range(70)]
+    for o in outs:
+        call(wc, kic, qc, kc, vc, o)
+    torch.cuda.synchronize()
+    del ki
+    ki = plan(wb)
+    print(f"[case] block tables of the new plan at the old addresses: {[t.data_ptr() for t in ki.block_tables] == addresses}", flush=True)
+    qb, kb, vb = wb.tensors(dev)
+    out = torch.full_like(qb, float("nan"))
+    lse = None
+    call(wb, ki, qb, kb, vb, out)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(wb, qb, kb, vb)
+    err = (out.float().cpu() - ref_out.float()).abs().max().item()
+    assert err <= TOL[wb.dtype], f"new plan at recycled addresses: output error {err}"
