@@ -223,6 +223,11 @@ typedef struct pat_fwd_bucket {
   const int32_t* kv;          /* [num_boxes]                                  */
   const int32_t* q_slot;      /* optional [num_boxes, q_table_stride] (see     */
                               /* pat_bucket_view.q_slot); NULL: use CTA_rank   */
+  /* Filing by CTA_rank (q_slot NULL) is what the reference does and is right only where every
+   * sequence's boxes carry the ranks 0 .. num_split_per_seq - 1, each once (regular trees). Where
+   * the scheduler repeats or skips a rank within a sequence (irregular forests), one partial
+   * result overwrites another or the merge reads a slot nobody wrote: pass the planner's q_slot
+   * and num_boxes_per_seq, or derive both on the device with pat_fwd_derive_slots. */
   int64_t q_table_stride;     /* elements between rows                        */
   int64_t block_table_stride; /* elements between rows                        */
   int32_t num_boxes;
@@ -352,7 +357,7 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
  * space than the array holds fails with PAT_ERR_WORKSPACE and enqueues nothing. Every call on a GPU
  * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls
  * on one stream are ordered and safe. Nothing in the array has to be cleared between calls: every
- * slot a call reads it writes first. */
+ * slot a call reads it writes first (slots filed as described at pat_fwd_bucket.q_slot). */
 int pat_fwd_launch_static(const pat_fwd_args* args, void* hip_stream);
 size_t pat_fwd_static_scratch_bytes(void);
 

@@ -633,10 +633,10 @@ __global__ void __launch_bounds__(256) pat_slot_kernel(const SlotParams p) {
     for (int base = 0; base < entries; base += 64) {
       const int e = base + lane;
       bool live = false, hit = false;
-      int at = 0;
+      int64_t at = 0;
       if (e < entries) {
         const int box = e / bk.max_seqs, j = e - box * bk.max_seqs;
-        at = box * bk.q_stride + j;
+        at = (int64_t)box * bk.q_stride + j;
         const int q = bk.q_table[at];
         live = j < bk.num_seqs[box] && (unsigned)q < (unsigned)p.batch;
         hit = live && q == s;

@@ -65,6 +65,8 @@ c10::Device to_device(const py::object& obj) {
   return obj.cast<c10::Device>();
 }
 
+struct RecordSet;
+
 // ---- a prepared launch ------------------------------------------------------------------------
 // pat_fwd_args plus everything it points into. Built once per set of tensors (a decode step calls
 // the forward once per layer with the same plan), launched many times.
@@ -72,7 +74,7 @@ struct Prepared {
   pat_fwd_args args;
   std::vector<pat_fwd_bucket> buckets;
   TensorList keep;          // plan tensors (and derived slots) stay alive as long as the launch does
-  at::Tensor records;       // the plan's launch records (shared by every launch of the plan)
+  std::shared_ptr<RecordSet> records;   // the plan's launch records (shared by every launch of the plan)
   int64_t plan_version = -1;   // version of the plan tables the records were built from
   size_t need = 0;          // workspace bytes
   pat_fwd_tuning tuning;    // the measured geometry of this plan shape (args.tuning points here when set)
@@ -115,10 +117,9 @@ void tune(Prepared& L, const c10::Device& dev) {
     auto it = g_tuned.find(key);
     if (it != g_tuned.end()) { L.tuning = it->second; L.args.tuning = &L.tuning; return; }
   }
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   void* stream = static_cast<void*>(c10::hip::getCurrentHIPStream(dev.index()).stream());
-  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess ||
-      capturing != hipStreamCaptureStatusNone)
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
     return;
   size_t most = 0;
   check(pat_fwd_autotune_workspace_bytes(&L.args, &most));
@@ -152,9 +153,28 @@ void tune(Prepared& L, const c10::Device& dev) {
 // The records depend on the plan tables and the launch geometry, not on q / k / v / out: the layers
 // of a model (one prepared launch each) share one set. `version` counts in-place edits of the plan
 // tables (torch's version counter): records of an older version are dropped.
+// One set of records: the tensor, and an event recorded behind the kernel that wrote it. A launch
+// on another stream than the one that built the records waits for that event (torch orders work
+// per stream only, and this tensor is not the caller's to synchronise).
+struct RecordSet {
+  at::Tensor tensor;
+  hipEvent_t ready = nullptr;   // null: built while the stream was being captured (ordered inside that graph)
+  void* stream = nullptr;       // the stream that built them
+  bool seen_ready = false;
+  RecordSet() = default;
+  RecordSet(const RecordSet&) = delete;
+  RecordSet& operator=(const RecordSet&) = delete;
+  ~RecordSet() { if (ready != nullptr) (void)hipEventDestroy(ready); }
+};
+
+bool capturing(void* stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  return hipStreamIsCapturing(static_cast<hipStream_t>(stream), &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+}
+
 struct RecordStore {
   int64_t version = -1;
-  std::unordered_map<uint64_t, at::Tensor> by_tag;
+  std::unordered_map<uint64_t, std::shared_ptr<RecordSet>> by_tag;
   // plans that came without slot tables: the ordinals derived on the device (pat_fwd_derive_slots)
   at::Tensor derived_slots;
   std::vector<int64_t> derived_offsets;
@@ -174,16 +194,24 @@ void attach_records(Prepared& L, RecordStore& store, int64_t version, const c10:
   if (it == store.by_tag.end()) {
     size_t rbytes = 0;
     check(pat_fwd_records_bytes(&a, &rbytes));
-    at::Tensor records = at::empty({(int64_t)rbytes}, at::TensorOptions().dtype(at::kByte).device(dev));
+    auto set = std::make_shared<RecordSet>();
+    set->tensor = at::empty({(int64_t)rbytes}, at::TensorOptions().dtype(at::kByte).device(dev));
+    set->stream = raw_stream(dev);
     uint64_t built = 0;
-    check(pat_fwd_build_records(&a, records.data_ptr(), rbytes, &built, raw_stream(dev)));
+    // (the derived slots of a plan without slot tables were written on this stream just before: the
+    // event covers them too)
+    check(pat_fwd_build_records(&a, set->tensor.data_ptr(), rbytes, &built, set->stream));
+    if (!capturing(set->stream)) {
+      require(hipEventCreateWithFlags(&set->ready, hipEventDisableTiming) == hipSuccess, "hipEventCreateWithFlags failed");
+      require(hipEventRecord(set->ready, static_cast<hipStream_t>(set->stream)) == hipSuccess, "hipEventRecord failed");
+    }
     if (store.by_tag.size() >= 16) store.by_tag.clear();
-    it = store.by_tag.emplace(built, records).first;
+    it = store.by_tag.emplace(built, set).first;
     tag = built;
   }
   L.records = it->second;
   L.plan_version = version;
-  a.records = L.records.data_ptr(); a.records_bytes = (size_t)L.records.numel(); a.records_tag = tag;
+  a.records = L.records->tensor.data_ptr(); a.records_bytes = (size_t)L.records->tensor.numel(); a.records_tag = tag;
   check(pat_fwd_workspace_bytes(&a, &L.need));
 }
 
@@ -319,7 +347,16 @@ void run(Prepared& L, const c10::Device& dev) {
     L.args.workspace = nullptr;
   }
   L.args.workspace_bytes = L.need;
-  check(pat_fwd_launch(&L.args, raw_stream(dev)));
+  void* stream = raw_stream(dev);
+  if (L.records && L.records->ready != nullptr && !L.records->seen_ready && stream != L.records->stream &&
+      !capturing(stream)) {
+    // another stream than the one that wrote the records: ordered behind that kernel (not while
+    // this stream is being captured, where events of the outside world may not be touched: a capture
+    // follows a warm-up call and a synchronisation, which is what orders it)
+    if (hipEventQuery(L.records->ready) == hipSuccess) L.records->seen_ready = true;
+    else require(hipStreamWaitEvent(static_cast<hipStream_t>(stream), L.records->ready, 0) == hipSuccess, "hipStreamWaitEvent failed");
+  }
+  check(pat_fwd_launch(&L.args, stream));
 }
 
 // ---- cache keys -----------------------------------------------------------------------------------

@@ -906,3 +906,31 @@ def test_table_form_new_plan_at_recycled_addresses():
     ref_out, ref_lse = _oracle(wb, qb, kb, vb)
     err = (out.float().cpu() - ref_out.float()).abs().max().item()
     assert err <= TOL[wb.dtype], f"new plan at recycled addresses: output error {err}"
+
+
+def test_launches_of_one_plan_from_two_streams():
+    # What the binding builds per plan (launch records) is written by a kernel on the stream of the
+    # first call; a call on another stream right behind it must be ordered after that kernel.
+    print("[case] one plan, first call on one stream, second on another", flush=True)
+    dev = _device()
+    w = workloads.make("c3", seed=1)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    out1, out2 = torch.full_like(q, float("nan")), torch.full_like(q, float("nan"))
+    lse1 = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    lse2 = lse1.clone()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out1, softmax_lse=lse1)
+    with torch.cuda.stream(s2):
+        prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out2, softmax_lse=lse2)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("two streams, first", out1, lse1, ref_out, ref_lse, w.dtype)
+    _assert_close("two streams, second", out2, lse2, ref_out, ref_lse, w.dtype)
+    assert torch.equal(out1, out2)
