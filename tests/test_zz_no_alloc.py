@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (pat_fwd_launch_static) against pat_fwd_launch, through
 the C ABI: same kernels, the partial results in the library's built-in scratch array instead of a
 caller's workspace. Two calls in a row, the second on a smaller batch (the scratch keeps the first
-call's contents), bit-identical outputs required."""
+call's contents), bit-identical outputs required. Then the use it exists for: the call captured into
+a HIP graph and replayed, every replay against an eager pat_fwd_launch."""
 import ctypes as C
 import math
 
@@ -54,3 +55,51 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
     print("[case] pat_fwd_launch_static vs pat_fwd_launch: c2, then the smaller c1", flush=True)
     _both_routes("c2", workloads.make("c2", seed=0), dev)
     _both_routes("c1", workloads.make("c1", seed=0), dev)   # smaller: stale partial results stay behind it
+
+
+def test_static_scratch_entry_point_under_graph_capture():
+    # what the entry point is for: a caller that captures the call into a HIP graph (no allocation
+    # may happen there) and replays it; every replay against an eager pat_fwd_launch on the same inputs
+    assert torch.cuda.is_available(), "GPU tests need an AMD GPU"
+    dev = torch.device("cuda:0")
+    print("[case] pat_fwd_launch_static captured into a HIP graph and replayed, c2", flush=True)
+    lib = _lib.load()
+    w = workloads.make("c2", seed=3)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    lt = info.launch_tables()
+    q_static = q.clone()
+    out_graph = torch.zeros_like(q)
+    out_eager = torch.zeros_like(q)
+
+    def prepared(qq, oo):
+        return _ctypes_launch.prepare(qq, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"],
+                                      lt["num_seqs_per_CTAs"], lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"],
+                                      info.max_boxes_per_seq, info.max_seqs_in_CTA, info.max_blocks_in_CTA,
+                                      1.0 / math.sqrt(w.head_dim), oo, None, lt["slot_tables"], lt.get("flags"))
+
+    Lg, Le = prepared(q_static, out_graph), prepared(q_static, out_eager)
+    Lg.args.workspace, Lg.args.workspace_bytes = None, 0
+    ws = torch.empty(Le.need, dtype=torch.uint8, device=dev)
+    Le.args.workspace, Le.args.workspace_bytes = ws.data_ptr(), Le.need
+    # first call outside the capture (it looks up the scratch array's address once per device)
+    assert lib.pat_fwd_launch_static(C.byref(Lg.args), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)) == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.pat_fwd_launch_static(C.byref(Lg.args), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    assert rc == 0, _lib.last_error()
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    for trial in range(3):
+        q_static.copy_(torch.randn(q.shape, generator=gen).to(w.dtype).to(dev))
+        out_graph.fill_(float("nan"))
+        out_eager.fill_(float("nan"))
+        assert lib.pat_fwd_launch(C.byref(Le.args), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)) == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph, out_eager), f"replay {trial} differs from the eager call"
