@@ -77,7 +77,10 @@ def build(jobs: int = 4, verbose: bool = False) -> str:
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         objs: List[str] = list(pool.map(lambda s: _compile(s, verbose), SOURCES))
     tmp = OUT + ".tmp"
-    cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", tmp, *objs]
+    # No RUNPATH to the ROCm the library was built with: a process has ONE HIP runtime. Where torch is
+    # loaded, its own libamdhip64 (same SONAME) serves this library too; elsewhere the loader's
+    # configured search path (ld.so.conf / LD_LIBRARY_PATH) finds the system's.
+    cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-rtlib-add-rpath", "-o", tmp, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -111,8 +114,10 @@ def build_extension(verbose: bool = False) -> str:
            "-DTORCH_EXTENSION_NAME=_prefix_attn", "-DTORCH_API_INCLUDE_EXTENSION_H",
            *[f"-isystem{p}" if "torch" in p or "rocm" in p else f"-I{p}" for p in includes],
            EXT_SRC, "-o", tmp,
-           f"-L{HERE}", "-lpat_amd", f"-L{torch_lib}", "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
-           "-lc10", "-lc10_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+           # torch's libraries come before libpat_amd in the dependency list: the loader then maps
+           # torch's HIP runtime first and resolves libpat_amd's libamdhip64.so.7 to that same object
+           f"-L{torch_lib}", "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+           f"-L{HERE}", "-lpat_amd", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -3,7 +3,10 @@
 //    same reductions with __shfl_xor;
 //  * ds_read_b64_tr_b16: within a 16-lane group, result lane i element r is source lane
 //    (4r + i/4) element (i%4), the mapping the transposed V reads are addressed for.
-// Both were established on the hardware; a compiler or driver that breaks one of them shows up
+//  * v_mfma_f32_32x32x16_f16: A lane l holds row l%32, k = 8(l/32)..+7; B lane l holds column l%32,
+//    k = 8(l/32)..+7; accumulator register i of lane l is element (8(i/4) + 4(l/32) + i%4, l%32):
+//    the layouts the tall-box path of the split kernel is written for.
+// All were established on the hardware; a compiler or driver that breaks one of them shows up
 // here instead of as wrong attention outputs.
 #include <hip/hip_runtime.h>
 
@@ -15,6 +18,8 @@ namespace pat {
 namespace {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 __global__ void selftest_kernel(int* failures) {
   __shared__ __attribute__((aligned(16))) short tile[64 * 4];
@@ -43,6 +48,29 @@ __global__ void selftest_kernel(int* failures) {
   for (int r = 0; r < 4; ++r) {
     const int src_lane = grp + 4 * r + i / 4;
     bad += got[r] != (short)(src_lane * 4 + (i % 4));
+  }
+  // ---- 32x32x16 MFMA operand and accumulator layouts ----------------------------------------
+  {
+    auto A = [](int m, int k) { return (float)((m * 3 + k * 5) % 7 - 3); };
+    auto B = [](int k, int c) { return (float)((k * 2 + c) % 5 - 2); };
+    const int half = lane >> 5, idx = lane & 31;
+    f16x8 a, b;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      a[j] = (_Float16)A(idx, 8 * half + j);
+      b[j] = (_Float16)B(8 * half + j, idx);
+    }
+    f32x16 c;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c[r] = 0.f;
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = 8 * (r / 4) + 4 * half + r % 4;
+      float want = 0.f;
+      for (int k = 0; k < 16; ++k) want += A(m, k) * B(k, idx);
+      bad += c[r] != want;
+    }
   }
   if (bad) atomicAdd(failures, bad);
 }

@@ -12,6 +12,7 @@
 #include <torch/extension.h>
 
 #include <c10/core/DeviceGuard.h>
+#include <c10/core/InferenceMode.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 
@@ -76,7 +77,9 @@ struct Prepared {
   TensorList keep;          // plan tensors (and derived slots) stay alive as long as the launch does
   std::shared_ptr<RecordSet> records;   // the plan's launch records (shared by every launch of the plan)
   int64_t plan_version = -1;   // version of the plan tables the records were built from
-  size_t need = 0;          // workspace bytes
+  size_t need = 0;          // workspace bytes with prebuilt records
+  size_t need_inline = 0;   // workspace bytes when the launch builds its records itself (args.records NULL)
+  bool derive_slots = false;   // the plan came without slot tables: ordinals derived on the device
   pat_fwd_tuning tuning;    // the measured geometry of this plan shape (args.tuning points here when set)
   Prepared() { std::memset(&args, 0, sizeof(args)); std::memset(&tuning, 0, sizeof(tuning)); }
 };
@@ -89,9 +92,12 @@ struct Prepared {
 // rounded up to multiples of 8.
 std::mutex g_tune_mutex;
 std::unordered_map<std::string, pat_fwd_tuning> g_tuned;
+// Opt-in (PAT_AUTOTUNE=1 or set_autotune(True)): the measurement synchronises the stream and runs
+// the launch some fifty times, which a serving loop must not meet unasked; the automatic geometry
+// (sizes only) is the default.
 bool g_autotune = [] {
   const char* e = std::getenv("PAT_AUTOTUNE");
-  return e == nullptr || std::atoi(e) != 0;
+  return e != nullptr && std::atoi(e) != 0;
 }();
 
 std::string shape_key(const pat_fwd_args& a) {
@@ -151,14 +157,23 @@ void tune(Prepared& L, const c10::Device& dev) {
 
 // ---- launch records, shared by the launches of one plan -----------------------------------------
 // The records depend on the plan tables and the launch geometry, not on q / k / v / out: the layers
-// of a model (one prepared launch each) share one set. `version` counts in-place edits of the plan
-// tables (torch's version counter): records of an older version are dropped.
+// of a model (one prepared launch each) share one set. They are a SNAPSHOT of the tables, taken when
+// a launch first needs them and again when torch's version counter of a plan tensor has moved
+// (in-place edits through torch: DecodePlan.advance_step). Edits torch does not count are not seen:
+//   * while the stream is being captured into a graph no snapshot is used: the launch builds its
+//     records itself (args.records NULL), so the record kernel is part of the graph and every replay
+//     reads the tables as they are then;
+//   * a plan held in inference tensors (no version counter) is served the same way at every call;
+//   * anything else (raw-pointer writes by another library): KernelInfo.invalidate() /
+//     invalidate_plans() drop the snapshots.
 // One set of records: the tensor, and an event recorded behind the kernel that wrote it. A launch
 // on another stream than the one that built the records waits for that event (torch orders work
 // per stream only, and this tensor is not the caller's to synchronise).
+constexpr int64_t kUntracked = -2;   // plan version of tensors without a version counter
+
 struct RecordSet {
   at::Tensor tensor;
-  hipEvent_t ready = nullptr;   // null: built while the stream was being captured (ordered inside that graph)
+  hipEvent_t ready = nullptr;
   void* stream = nullptr;       // the stream that built them
   bool seen_ready = false;
   RecordSet() = default;
@@ -178,12 +193,13 @@ struct RecordStore {
   // plans that came without slot tables: the ordinals derived on the device (pat_fwd_derive_slots)
   at::Tensor derived_slots;
   std::vector<int64_t> derived_offsets;
-  int64_t derived_version = -1;
+  int64_t derived_version = -1;   // plan version whose ordinals the buffer holds (-1: none that may be relied on)
   // a store looked up by the plan tensors' addresses holds those tensors: as long as it exists no
   // other plan can be allocated at the same addresses and find records that are not its own
   TensorList keep;
 };
 
+// Snapshot of the plan at `version` for this launch; never called while the stream is being captured.
 void attach_records(Prepared& L, RecordStore& store, int64_t version, const c10::Device& dev) {
   if (store.version != version) { store.by_tag.clear(); store.version = version; }
   pat_fwd_args& a = L.args;
@@ -201,10 +217,8 @@ void attach_records(Prepared& L, RecordStore& store, int64_t version, const c10:
     // (the derived slots of a plan without slot tables were written on this stream just before: the
     // event covers them too)
     check(pat_fwd_build_records(&a, set->tensor.data_ptr(), rbytes, &built, set->stream));
-    if (!capturing(set->stream)) {
-      require(hipEventCreateWithFlags(&set->ready, hipEventDisableTiming) == hipSuccess, "hipEventCreateWithFlags failed");
-      require(hipEventRecord(set->ready, static_cast<hipStream_t>(set->stream)) == hipSuccess, "hipEventRecord failed");
-    }
+    require(hipEventCreateWithFlags(&set->ready, hipEventDisableTiming) == hipSuccess, "hipEventCreateWithFlags failed");
+    require(hipEventRecord(set->ready, static_cast<hipStream_t>(set->stream)) == hipSuccess, "hipEventRecord failed");
     if (store.by_tag.size() >= 16) store.by_tag.clear();
     it = store.by_tag.emplace(built, set).first;
     tag = built;
@@ -318,15 +332,23 @@ std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, cons
   }
   if (slots == nullptr && max_split > 1) {
     // A plan without slot tables (the reference's call form): CTA_rank is not unique per sequence on
-    // irregular forests, so the ordinals are derived from the q_tables on the device, once per
-    // prepared launch (the caches key on the tables' version counters).
-    if (!store.derived_slots.defined() || store.derived_version != plan_version) {
+    // irregular forests, so the ordinals are derived from the q_tables on the device: once per plan
+    // version here or in run(), at every call where no snapshot may be used.
+    L->derive_slots = true;
+    if (!store.derived_slots.defined()) {
       size_t sbytes = 0;
       check(pat_fwd_slots_bytes(&a, &sbytes));
       store.derived_slots = at::empty({(int64_t)sbytes}, at::TensorOptions().dtype(at::kByte).device(q.device()));
       store.derived_offsets.assign(std::max<size_t>(nb, 1), 0);
-      check(pat_fwd_derive_slots(&a, store.derived_slots.data_ptr(), sbytes, store.derived_offsets.data(), raw_stream(q.device())));
-      store.derived_version = plan_version;
+      store.derived_version = -1;
+    }
+    void* stream = raw_stream(q.device());
+    const bool snapshot = plan_version != kUntracked && !capturing(stream);
+    if (!snapshot || store.derived_version != plan_version) {
+      // (also what fills derived_offsets, which is host arithmetic)
+      check(pat_fwd_derive_slots(&a, store.derived_slots.data_ptr(), (size_t)store.derived_slots.numel(),
+                                 store.derived_offsets.data(), stream));
+      store.derived_version = snapshot ? plan_version : -1;
     }
     int32_t* base = static_cast<int32_t*>(store.derived_slots.data_ptr());
     for (size_t i = 0; i < nb; ++i) L->buckets[i].q_slot = base + store.derived_offsets[i];
@@ -334,29 +356,45 @@ std::shared_ptr<Prepared> prepare(const at::Tensor& q, const at::Tensor& k, cons
     L->keep.push_back(store.derived_slots);
   }
   tune(*L, q.device());
-  attach_records(*L, store, plan_version, q.device());
+  a.records = nullptr; a.records_bytes = 0;
+  check(pat_fwd_workspace_bytes(&a, &L->need_inline));
   return L;
 }
 
-void run(Prepared& L, const c10::Device& dev) {
-  at::Tensor ws;   // scratch for the partial results (none for a single-slot launch); stream-ordered reuse
-  if (L.need > 0) {
-    ws = at::empty({(int64_t)L.need}, at::TensorOptions().dtype(at::kByte).device(dev));
-    L.args.workspace = ws.data_ptr();
-  } else {
-    L.args.workspace = nullptr;
-  }
-  L.args.workspace_bytes = L.need;
+void run(Prepared& L, RecordStore& store, int64_t version, const c10::Device& dev) {
   void* stream = raw_stream(dev);
-  if (L.records && L.records->ready != nullptr && !L.records->seen_ready && stream != L.records->stream &&
-      !capturing(stream)) {
-    // another stream than the one that wrote the records: ordered behind that kernel (not while
-    // this stream is being captured, where events of the outside world may not be touched: a capture
-    // follows a warm-up call and a synchronisation, which is what orders it)
-    if (hipEventQuery(L.records->ready) == hipSuccess) L.records->seen_ready = true;
-    else require(hipStreamWaitEvent(static_cast<hipStream_t>(stream), L.records->ready, 0) == hipSuccess, "hipStreamWaitEvent failed");
+  const bool snapshot = version != kUntracked && !capturing(stream);
+  pat_fwd_args& a = L.args;
+  if (L.derive_slots && (!snapshot || store.derived_version != version)) {
+    std::vector<int64_t> offsets(store.derived_offsets.size(), 0);
+    a.records = nullptr;
+    check(pat_fwd_derive_slots(&a, store.derived_slots.data_ptr(), (size_t)store.derived_slots.numel(), offsets.data(), stream));
+    store.derived_version = snapshot ? version : -1;
   }
-  check(pat_fwd_launch(&L.args, stream));
+  size_t need;
+  if (snapshot) {
+    if (!L.records || L.plan_version != version) attach_records(L, store, version, dev);
+    a.records = L.records->tensor.data_ptr(); a.records_bytes = (size_t)L.records->tensor.numel();
+    need = L.need;
+    if (!L.records->seen_ready && stream != L.records->stream) {
+      // another stream than the one that wrote the records: ordered behind that kernel
+      if (hipEventQuery(L.records->ready) == hipSuccess) L.records->seen_ready = true;
+      else require(hipStreamWaitEvent(static_cast<hipStream_t>(stream), L.records->ready, 0) == hipSuccess, "hipStreamWaitEvent failed");
+    }
+  } else {
+    // no snapshot: the launch builds its records from the tables as they are when it runs
+    a.records = nullptr; a.records_bytes = 0;
+    need = L.need_inline;
+  }
+  at::Tensor ws;   // scratch for the partial results (and inline records); stream-ordered reuse
+  if (need > 0) {
+    ws = at::empty({(int64_t)need}, at::TensorOptions().dtype(at::kByte).device(dev));
+    a.workspace = ws.data_ptr();
+  } else {
+    a.workspace = nullptr;
+  }
+  a.workspace_bytes = need;
+  check(pat_fwd_launch(&a, stream));
 }
 
 // ---- cache keys -----------------------------------------------------------------------------------
@@ -369,7 +407,7 @@ struct Key {
     for (int64_t s : t.strides()) add(s);
   }
   void plan_tensor(const at::Tensor& t) {   // ... and the version counter: in-place edits of a plan count
-    tensor(t); add((int64_t)t._version());
+    tensor(t); add(t.is_inference() ? kUntracked : (int64_t)t._version());
   }
 };
 
@@ -397,13 +435,21 @@ struct KernelInfo {
 
   // Counts in-place edits of the plan tables: every table is a view of one buffer, whose version
   // counter torch advances with each of them (a plan held table by table: the counters' sum).
+  // kUntracked when a table is an inference tensor (no counter). invalidate() moves it by hand.
+  int64_t generation = 0;
   int64_t plan_version() const {
-    if (flat.has_value()) return (int64_t)flat->_version();
-    int64_t v = (int64_t)num_split_per_seq._version() + (int64_t)num_boxes_per_seq._version();
+    const int64_t gen = generation << 32;
+    if (flat.has_value()) return flat->is_inference() ? kUntracked : gen + (int64_t)flat->_version();
+    if (num_split_per_seq.is_inference() || num_boxes_per_seq.is_inference()) return kUntracked;
+    int64_t v = gen + (int64_t)num_split_per_seq._version() + (int64_t)num_boxes_per_seq._version();
     for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables})
-      for (const at::Tensor& t : *l) v += (int64_t)t._version();
+      for (const at::Tensor& t : *l) {
+        if (t.is_inference()) return kUntracked;
+        v += (int64_t)t._version();
+      }
     return v;
   }
+  void invalidate() { ++generation; }
 
   void clear_tables() {
     for (TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables, &l_q_tables,
@@ -452,6 +498,9 @@ struct KernelInfo {
   // Copies every plan tensor to `device`: one copy of the one buffer, asynchronous from pinned memory
   // (the reference moves each table by itself, csrc/prefix_tree.h:27-38).
   void to_gpu(const c10::Device& device) {
+    // (plan tensors are ordinary tensors also when the caller is in inference mode: their version
+    // counters are what tells a launch that DecodePlan.advance_step edited them)
+    c10::InferenceMode plain(false);
     if (flat.has_value()) {
       flat = flat->to(device, /*non_blocking=*/true);
       bind(*flat);
@@ -566,6 +615,7 @@ struct PrefixTreeCPP {
       if (rc == PAT_OK) rc_flat = pat_tree_flat_plan(native->h, &fresh->layout, nullptr, 0);
     }
     check(rc);
+    c10::InferenceMode plain(false);   // plan tensors keep their version counters (see KernelInfo::to_gpu)
     if (rc_flat == PAT_OK) {
       const int64_t total = std::max<int64_t>(fresh->layout.total, 1);
       host = at::empty({total}, at::TensorOptions().dtype(at::kInt).pinned_memory(at::hasHIP() || at::hasCUDA()));
@@ -648,21 +698,37 @@ void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, c
   key.add(scale);
   key.bytes += plan_key.bytes;
 
+  // (version counters are part of the key: an edited plan is another key; tensors without a counter
+  // are served without snapshots)
+  bool tracked = !num_split.is_inference();
+  for (const TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs})
+    for (const at::Tensor& t : *l) tracked = tracked && !t.is_inference();
+  if (slot_tables.has_value()) for (const at::Tensor& t : *slot_tables) tracked = tracked && !t.is_inference();
+  const int64_t version = tracked ? 0 : kUntracked;
+
   std::shared_ptr<Prepared> L;
+  std::shared_ptr<RecordStore> store;
   {
     std::lock_guard<std::mutex> lock(g_table_mutex);
     auto it = g_table_launches.find(key.bytes);
-    if (it != g_table_launches.end()) L = it->second;
+    if (it != g_table_launches.end()) {
+      L = it->second;
+      auto st = g_table_records.find(plan_key.bytes);
+      if (st != g_table_records.end()) store = st->second; else L.reset();
+    }
   }
   if (!L) {
     PlanTables pt{&q_tables, &block_tables, &num_seqs, &ranks, &kvs,
                   slot_tables.has_value() ? &*slot_tables : nullptr, &mnw,
                   bucket_flags.has_value() ? &*bucket_flags : nullptr};
     // the launch records belong to the plan (tables + their versions), not to q / k / v / out
-    std::shared_ptr<RecordStore> store;
     {
       std::lock_guard<std::mutex> lock(g_table_mutex);
-      if (g_table_records.size() >= 16) g_table_records.clear();
+      // (launches hold pointers into their plan's store: both maps are emptied together)
+      if (g_table_records.size() >= 16 && g_table_records.find(plan_key.bytes) == g_table_records.end()) {
+        g_table_records.clear();
+        g_table_launches.clear();
+      }
       auto& slot = g_table_records[plan_key.bytes];
       if (!slot) {
         slot = std::make_shared<RecordStore>();
@@ -673,12 +739,12 @@ void fwd_tables(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, c
       }
       store = slot;
     }
-    L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse, *store, 0);
+    L = prepare(q, k, v, num_split, pt, max_split, max_seqs, max_blocks, scale, out, lse, *store, version);
     std::lock_guard<std::mutex> lock(g_table_mutex);
     if (g_table_launches.size() >= 64) g_table_launches.clear();
     g_table_launches[key.bytes] = L;
   }
-  run(*L, q.device());
+  run(*L, *store, version, q.device());
 }
 
 void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, PrefixTreeCPP& tree, double scale,
@@ -694,9 +760,7 @@ void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, Pre
   const int64_t version = info.plan_version();
   auto it = info.cache.find(key.bytes);
   if (it != info.cache.end()) {
-    L = it->second;
-    // the plan tables were edited in place since (DecodePlan.advance_step): records of the new contents
-    if (L->plan_version != version) attach_records(*L, info.records, version, q.device());
+    L = it->second;   // (run() takes a new snapshot when the plan tables were edited in place since)
   } else {
     const bool l = info.has_launch;
     const std::vector<int> no_flags;
@@ -712,7 +776,7 @@ void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, Pre
     if (info.cache.size() >= 256) info.cache.clear();
     info.cache[key.bytes] = L;
   }
-  run(*L, q.device());
+  run(*L, info.records, version, q.device());
 }
 
 void paged_decode_baseline(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& block_table,
@@ -781,6 +845,9 @@ PYBIND11_MODULE(_prefix_attn, m) {
       .def_readonly("max_split_per_seq", &KernelInfo::max_split)
       .def_readonly("max_seqs_in_CTA", &KernelInfo::max_seqs)
       .def_readonly("max_blocks_in_CTA", &KernelInfo::max_blocks)
+      .def("invalidate", &KernelInfo::invalidate,
+           "Drops what launches remember about the plan tables' contents (launch records, derived slots): call it "
+           "after writing to the tables by means torch's version counters do not see.")
       .def("launch_tables", &KernelInfo::launch_tables,
            "The per-bucket tables as the kernels get them (boxes longest first, a bucket with a wide head split "
            "in two) with their tile labels under \"MNWs\" and hints under \"flags\".")
@@ -834,10 +901,17 @@ PYBIND11_MODULE(_prefix_attn, m) {
   m.def("prefix_attn_with_kvcache", &fwd_tree, py::arg("q"), py::arg("k_cache_paged"), py::arg("v_cache_paged"),
         py::arg("tree"), py::arg("softmax_scale"), py::arg("out"), py::kw_only(), py::arg("softmax_lse") = py::none(),
         "Tree form: the plan of a PrefixTreeCPP whose kernel_info is on the device.");
+  m.def("invalidate_plans", [] {
+          std::lock_guard<std::mutex> lock(g_table_mutex);
+          g_table_launches.clear();
+          g_table_records.clear();
+        },
+        "Table form: drops every remembered launch and plan snapshot (launch records, derived slots). For plan "
+        "tables written by means torch's version counters do not see.");
   m.def("set_autotune", [](bool on) { g_autotune = on; }, py::arg("enabled"),
-        "Measured choice of the launch geometry (pat_fwd_autotune) the first time a plan shape is launched: on by "
-        "default (PAT_AUTOTUNE=0 in the environment switches it off). The measurement runs the launch a few "
-        "times per candidate on the current stream and synchronises it once per shape.");
+        "Measured choice of the launch geometry (pat_fwd_autotune) the first time a plan shape is launched: off "
+        "unless switched on here or with PAT_AUTOTUNE=1. The measurement runs the launch some fifty times on the "
+        "current stream and synchronises it, once per shape.");
   m.def("get_autotune", [] { return g_autotune; });
   m.def("clear_autotune_cache", [] { std::lock_guard<std::mutex> lock(g_tune_mutex); g_tuned.clear(); });
   m.def("paged_decode_baseline", &paged_decode_baseline, py::arg("q"), py::arg("k_cache_paged"),

@@ -154,3 +154,22 @@ def test_planner_calls_release_the_gil():
     assert tree.kernel_info.num_split_per_seq.numel() == n
     # with the GIL held throughout, the other thread would get at most a few switches
     assert during > 20 or native_s < 0.005, (during, native_s)
+
+
+def test_plan_tensors_keep_version_counters_under_inference_mode():
+    """A plan packed under torch.inference_mode() is held in ordinary tensors: the binding tells
+    in-place edits of a plan (DecodePlan.advance_step) by their version counters, which inference
+    tensors do not have."""
+    import torch
+    from pat_amd import PrefixTreeCPP, workloads
+    w = workloads.make("c1", seed=0)
+    with torch.inference_mode():
+        tree = PrefixTreeCPP(w.page_size)
+        tree.build_radix_tree(w.seq_lens, w.padded_table())
+        tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+        flat = tree.kernel_info._flat
+        assert flat is not None and not flat.is_inference()
+        before = flat._version
+        tree.kernel_info.kv_in_CTAs[0][0] += 1      # a view of the one buffer
+        assert flat._version > before
+    assert not tree.kernel_info.kv_in_CTAs[0].is_inference()

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import attn_oracle as ao
-from pat_amd import PrefixTree, PrefixTreeCPP, prefix_attn_with_kvcache, workloads
+from pat_amd import PrefixTree, PrefixTreeCPP, _prefix_attn, prefix_attn_with_kvcache, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -934,3 +934,139 @@ def test_launches_of_one_plan_from_two_streams():
     _assert_close("two streams, first", out1, lse1, ref_out, ref_lse, w.dtype)
     _assert_close("two streams, second", out2, lse2, ref_out, ref_lse, w.dtype)
     assert torch.equal(out1, out2)
+
+
+def test_plans_built_under_inference_mode():
+    # a plan packed, moved and used under torch.inference_mode(): the tree's own tensors keep their
+    # version counters; a table-form plan of inference tensors (no counter) is served without
+    # snapshots of its contents, so an in-place edit is seen by the next call
+    print("[case] inference_mode: tree form and table form of inference tensors, c1", flush=True)
+    dev = _device()
+    w = workloads.make("c1", seed=3)
+    q, k, v = w.tensors(dev)
+    scale = 1.0 / math.sqrt(w.head_dim)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    with torch.inference_mode():
+        tree = PrefixTreeCPP(w.page_size)
+        tree.build_radix_tree(w.seq_lens, w.padded_table())
+        tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+        tree.kernel_info.to_gpu(dev)
+        assert not tree.kernel_info._flat.is_inference()
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+        prefix_attn_with_kvcache(q, k, v, tree, scale, out, softmax_lse=lse)
+        torch.cuda.synchronize()
+        _assert_close("tree form under inference_mode", out, lse, ref_out, ref_lse, w.dtype)
+
+        t = PrefixTree(w.page_size)
+        t.build_radix_tree(w.seq_lens, w.rows)
+        ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+        ki.to_tensor(device=dev)
+        assert ki.kv_in_CTAs[0].is_inference()
+
+        def call(o, l):
+            prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                                     ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                                     ki.max_blocks_in_CTA, scale, o, softmax_lse=l)
+        out.fill_(float("nan"))
+        call(out, lse)
+        torch.cuda.synchronize()
+        _assert_close("table form of inference tensors", out, lse, ref_out, ref_lse, w.dtype)
+        # every request loses its last token (an in-place edit torch does not count): the next call sees it
+        lens = [n - 1 for n in w.seq_lens]
+        for b in range(len(ki.kv_in_CTAs)):
+            leaf = ki.num_seqs_per_CTAs[b] == 1
+            ki.kv_in_CTAs[b] -= leaf.to(torch.int32)
+        call(out, lse)
+        torch.cuda.synchronize()
+    ref2, ref2_lse = ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, lens, scale)
+    _assert_close("table form after an uncounted edit", out, lse, ref2, ref2_lse, w.dtype)
+
+
+def test_graph_replay_reads_the_plan_tables_of_the_moment():
+    # a captured call builds its launch records inside the graph: a replay after the plan tables
+    # were rewritten (here by a captured copy_, which no version counter sees from the launch's side)
+    # computes what an eager call on the same tables computes
+    print("[case] HIP graph whose plan tables change between replays, c1-shaped", flush=True)
+    dev = _device()
+    w = workloads.make("c1", seed=4)
+    q, k, v = w.tensors(dev)
+    scale = 1.0 / math.sqrt(w.head_dim)
+    t = PrefixTree(w.page_size)
+    t.build_radix_tree(w.seq_lens, w.rows)
+    ki = t.pack_schedule(MNWs=None, HRatio=w.heads // w.kv_heads, kvHead=w.kv_heads, use_compute_model=False)
+    ki.to_tensor(device=dev)
+    kv_full = [x.clone() for x in ki.kv_in_CTAs]
+    kv_short = [x - (n == 1).to(torch.int32) * 5 for x, n in zip(ki.kv_in_CTAs, ki.num_seqs_per_CTAs)]   # leaves lose 5 tokens
+    staged = [x.clone() for x in ki.kv_in_CTAs]
+    out_graph = torch.zeros_like(q)
+
+    def call(o):
+        prefix_attn_with_kvcache(q, k, v, ki.num_split_per_seq, ki.q_tables, ki.block_tables, ki.num_seqs_per_CTAs,
+                                 ki.CTA_ranks, ki.kv_in_CTAs, ki.MNWs, ki.max_split_per_seq, ki.max_seqs_in_CTA,
+                                 ki.max_blocks_in_CTA, scale, o)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(out_graph)                                                     # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for dst, src in zip(ki.kv_in_CTAs, staged):
+            dst.copy_(src)
+        call(out_graph)
+    for trial, (kvs, lens) in enumerate([(kv_short, [n - 5 for n in w.seq_lens]), (kv_full, list(w.seq_lens)),
+                                         (kv_short, [n - 5 for n in w.seq_lens])]):
+        for dst, src in zip(staged, kvs):
+            dst.copy_(src)
+        out_graph.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref_out, _ = ao.paged_attention_ref(q.cpu(), k.cpu(), v.cpu(), w.rows, lens, scale)
+        err = (out_graph.float().cpu() - ref_out.float()).abs().max().item()
+        print(f"[parity] replay {trial}: max|out - ref| = {err:.3e}", flush=True)
+        assert err <= TOL[w.dtype], f"replay {trial}: {err}"
+        out_eager = torch.full_like(q, float("nan"))
+        # (an eager call works from a snapshot of the tables taken per version counter; the replay's
+        # copy_ moved no counter, so the snapshots are dropped by hand)
+        _prefix_attn.invalidate_plans()
+        call(out_eager)                                                     # eager, same table contents
+        torch.cuda.synchronize()
+        assert torch.equal(out_eager, out_graph), f"replay {trial} differs from the eager call"
+
+
+def test_first_call_under_capture_then_eager():
+    # a launch whose very first call is captured (nothing but the capture's own pool has seen it)
+    # and is then called eagerly before any replay: the eager call builds its own launch records
+    print("[case] first call captured, then eager, c1", flush=True)
+    dev = _device()
+    w = workloads.make("c1", seed=5)
+    q, k, v = w.tensors(dev)
+    scale = 1.0 / math.sqrt(w.head_dim)
+    warm = workloads.make("c1", seed=6)
+    wq, wk, wv = warm.tensors(dev)
+    wtree = PrefixTreeCPP(warm.page_size)
+    wtree.build_radix_tree(warm.seq_lens, warm.padded_table())
+    wtree.pack_schedule(None, warm.heads // warm.kv_heads, warm.kv_heads)
+    wtree.kernel_info.to_gpu(dev)
+    prefix_attn_with_kvcache(wq, wk, wv, wtree, scale, torch.empty_like(wq))   # the library itself is warm
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    tree.kernel_info.to_gpu(dev)
+    torch.cuda.synchronize()
+    out_graph = torch.zeros_like(q)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        prefix_attn_with_kvcache(q, k, v, tree, scale, out_graph)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, scale, out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("eager after a captured first call", out, lse, ref_out, ref_lse, w.dtype)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert (out_graph.float().cpu() - ref_out.float()).abs().max().item() <= TOL[w.dtype]
