@@ -5,13 +5,19 @@
 
 A step is one call of the hot path (pat_fwd_launch through the C ABI of libpat_amd: split
 kernel + merge kernel) on one decode batch of the named workload, with the plan already on
-the device. Synthetic, seeded N(0,1) inputs are resident in HBM before the timed region; the
-KV cache is rotated over several copies whose total size exceeds the 256 MB Infinity Cache so
-that consecutive steps cannot be served from it.
+the device, under the launch geometry the library chooses from sizes alone (what the drop-in call
+does by default). Synthetic, seeded N(0,1) inputs are resident in HBM before the timed region;
+the KV cache is rotated over several copies whose total size exceeds the 256 MB Infinity Cache
+so that consecutive steps cannot be served from it.
 
 Prints ONE JSON line. `value` is unique-KV bytes / time per call (GB/s); `ms_per_step` is the
-latency per call. `roofline` covers the split kernel (HBM-bound): algorithmic bytes = unique
-KV bytes of the batch, duration = mean split-kernel time from HIP events on the launch stream.
+latency per call: W warm-up steps, then the K timed steps between two synchronisations, repeated
+5 times; the median repetition is reported, `ms_per_step_spread` holds the fastest and slowest.
+`roofline` covers the split kernel (HBM-bound): algorithmic bytes = unique KV bytes of the batch,
+duration = mean split-kernel time from HIP events on the launch stream. `autotune` reports what
+the optional measured choice of the geometry (pat_fwd_autotune, off by default in the product)
+would give and what measuring costs; `records_build_us` the kernel that turns the plan tables into
+launch records once per plan; `plan_build_ms_host` the host planner in steady state.
 `cpu_baseline` times this repository's CPU restatement of the reference's PyTorch attention
 on the host cores. `api_us_per_call` is the same loop through the drop-in call
 `prefix_attn_with_kvcache(q, k, v, tree, scale, out)` of the compiled extension (workspace from
@@ -107,11 +113,17 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     q, ks, vs = w.tensors(dev, copies=copies)
     scale = 1.0 / math.sqrt(w.head_dim)
 
-    t0 = time.perf_counter()
-    tree = PrefixTreeCPP(w.page_size)
-    tree.build_radix_tree(w.seq_lens, w.padded_table())
-    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
-    plan_ms = (time.perf_counter() - t0) * 1e3
+    def plan():
+        t0 = time.perf_counter()
+        tree = PrefixTreeCPP(w.page_size)
+        tree.build_radix_tree(w.seq_lens, w.padded_table())
+        tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+        return tree, (time.perf_counter() - t0) * 1e3
+
+    _, plan_first_ms = plan()          # (the first call also pays for the pinned buffer pool)
+    plan_runs = sorted(plan()[1] for _ in range(5))
+    tree, _ = plan()
+    plan_ms = plan_runs[len(plan_runs) // 2]
     info = tree.kernel_info
     info.to_gpu(dev)
 
@@ -119,8 +131,8 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def prepare(plan_kw, slots, autotune):
-        # One measured geometry per plan (pat_fwd_autotune, what the drop-in call does the first time
-        # it sees a plan shape), shared by the launches over the rotated cache copies.
+        # `autotune`: one measured geometry per plan (pat_fwd_autotune), shared by the launches over the
+        # rotated cache copies; otherwise the geometry the library derives from sizes.
         launches, tuning = [], None
         for i in range(copies):
             L = _ctypes_launch.prepare(q, ks[i], vs[i], plan_kw["num_split_per_seq"], plan_kw["query_tables"],
@@ -141,7 +153,17 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
                   CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"], MNW=lt["MNWs"],
                   max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                   max_blocks_in_CTA=info.max_blocks_in_CTA, bucket_flags=lt.get("flags"))
-    pat_launches, pat_ws = prepare(pat_kw, lt["slot_tables"], not a.no_autotune)
+    pat_slots = lt["slot_tables"]
+    whole = info.whole_sequence_tables()
+    if whole is not None:
+        # a small batch of short requests: the drop-in call launches one work item per request (one kernel)
+        pat_kw = dict(num_split_per_seq=whole["num_split_per_seq"], query_tables=whole["q_tables"],
+                      block_tables=whole["block_tables"], num_seqs_per_CTAs=whole["num_seqs_per_CTAs"],
+                      CTA_ranks=whole["CTA_ranks"], kv_in_CTAs=whole["kv_in_CTAs"], MNW=whole["MNWs"],
+                      max_split_per_seq=whole["max_split_per_seq"], max_seqs_in_CTA=whole["max_seqs_in_CTA"],
+                      max_blocks_in_CTA=whole["max_blocks_in_CTA"], bucket_flags=None)
+        pat_slots = None
+    pat_launches, pat_ws = prepare(pat_kw, pat_slots, False)
 
     def step(launches, i):
         rc = lib.pat_fwd_launch(C.byref(launches[i % copies].args), C.c_void_p(stream))
@@ -167,9 +189,28 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
         torch.cuda.synchronize()
         return (time.perf_counter() - t) * 1e3 / steps
 
-    ms_per_step = timed(pat_launches, steps, warmup)
+    def timed_median(launches, steps, warmup, reps=5):
+        runs = sorted(timed(launches, steps, warmup) for _ in range(reps))
+        return runs[len(runs) // 2], runs[0], runs[-1]
+
     if a.kernel_loop_only:
-        return {"ms_per_step": ms_per_step, "steps": steps, "warmup": warmup}
+        return {"ms_per_step": timed(pat_launches, steps, warmup), "steps": steps, "warmup": warmup}
+    ms_per_step, ms_fastest, ms_slowest = timed_median(pat_launches, steps, warmup)
+
+    # the record kernel of this plan (once per plan, outside the timed loop): HIP-event time of 5 builds
+    rec_bytes = C.c_size_t(0)
+    lib.pat_fwd_records_bytes(C.byref(pat_launches[0].args), C.byref(rec_bytes))
+    rec_buf = torch.empty(max(rec_bytes.value, 256), dtype=torch.uint8, device=dev)
+    rec_tag = C.c_uint64(0)
+    rec_ev = [(hip.event(), hip.event()) for _ in range(5)]
+    for e0, e1 in rec_ev:
+        hip.record(e0, stream)
+        rc = lib.pat_fwd_build_records(C.byref(pat_launches[0].args), C.c_void_p(rec_buf.data_ptr()), rec_bytes.value,
+                                       C.byref(rec_tag), C.c_void_p(stream))
+        assert rc == 0, _lib.last_error()
+        hip.record(e1, stream)
+    torch.cuda.synchronize()
+    records_build_us = sorted(hip.ms(e0, e1) for e0, e1 in rec_ev)[2] * 1e3
 
     # per-kernel durations from HIP events on the launch stream (same step sequence)
     n_ev = min(steps, 100)
@@ -209,6 +250,7 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
         "steps": steps,
         "warmup": warmup,
         "ms_per_step": round(ms_per_step, 6),
+        "ms_per_step_spread": [round(ms_fastest, 6), round(ms_slowest, 6)],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -229,21 +271,38 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
                      "merge_mean": round((mean(merge_ms) - event_overhead_ms) * 1e3, 3),
                      "merge_interval_mean": round(mean(merge_ms) * 1e3, 3),
                      "event_overhead_per_interval": round(event_overhead_ms * 1e3, 3)},
+        "launched_as": "one work item per request" if whole is not None else "planned",
         "geometry": {"chunk_tokens": geo.chunk_tokens, "tall_chunk_tokens": geo.tall_chunk_tokens,
                      "chunks_per_rank": geo.chunks_per_rank, "workgroups": geo.num_workgroups},
         "plan_build_ms_host": round(plan_ms, 3),
-        # the measured choice of the launch geometry (made once per plan shape, outside the timed
-        # region, like the plan itself): overrides in pat_fwd_tuning's field order, null = none
-        "autotune": None if a.no_autotune else {
-            "chosen": (None if pat_launches[0].tuning is None else
-                       {f: getattr(pat_launches[0].tuning, f) for f, _ in _lib.FwdTuning._fields_}),
-            "tuning_run_us": {"chosen": round(pat_launches[0].tuned_us, 2), "automatic": round(pat_launches[0].auto_us, 2)}},
+        "plan_build_first_call_ms": round(plan_first_ms, 3),
+        "records_build_us": round(records_build_us, 2),
+        "autotune": None,
         "roofline": {"bound": "hbm", "kernel": "pat_split_kernel", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": None},
     }
 
     result["roofline"]["traffic"] = measured_traffic_bytes(workload, a.seed, int(geo.num_workgroups))
+
+    if not a.no_autotune:
+        # What the optional measured choice of the geometry would give (pat_fwd_autotune; off by default
+        # in the product: it synchronises the stream and runs the launch some fifty times), and what the
+        # measurement costs in wall time.
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        tuned_launches, tuned_ws = prepare(pat_kw, pat_slots, True)
+        torch.cuda.synchronize()
+        tune_ms = (time.perf_counter() - t) * 1e3
+        tuned_ms, _, _ = timed_median(tuned_launches, steps, warmup)
+        L0 = tuned_launches[0]
+        result["autotune"] = {
+            "chosen": {f: getattr(L0.tuning, f) for f, _ in _lib.FwdTuning._fields_},
+            "tuned_us_per_call": round(tuned_ms * 1e3, 3),
+            "untuned_us_per_call": round(ms_per_step * 1e3, 3),
+            "autotune_wall_ms": round(tune_ms, 2),
+            "tuning_run_us": {"chosen": round(L0.tuned_us, 2), "automatic": round(L0.auto_us, 2)}}
+        del tuned_launches, tuned_ws
 
     # the same steps through the drop-in call of the compiled extension (tree form): argument checks
     # and launch preparation are cached per (q, k, v, out), the workspace comes from torch's
@@ -263,8 +322,8 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     if not a.no_oblivious:
         ob = workloads.oblivious_plan(w, dev)
         ob_kw = {k: ob[k] for k in pat_kw}
-        ob_launches, ob_ws = prepare(ob_kw, None, not a.no_autotune)
-        ob_ms = timed(ob_launches, steps, warmup)
+        ob_launches, ob_ws = prepare(ob_kw, None, False)
+        ob_ms, _, _ = timed_median(ob_launches, steps, warmup, reps=3)
         result["oblivious_us_per_call"] = round(ob_ms * 1e3, 3)
         result["speedup_vs_oblivious"] = round(ob_ms / ms_per_step, 3)
 
@@ -300,7 +359,7 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-oblivious", action="store_true")
     ap.add_argument("--no-autotune", action="store_true",
-                    help="launch geometry from sizes alone, without the measured choice the drop-in call makes")
+                    help="skip the side measurement of what pat_fwd_autotune would choose (the headline never uses it)")
     ap.add_argument("--no-configs", action="store_true",
                     help="do not measure the other benchmark workloads beside the named one")
     ap.add_argument("--kernel-loop-only", action="store_true",

@@ -27,9 +27,10 @@ constexpr int kTargetWgsPerCU = 2;  // what fits at once: 2 workgroups of 4 wave
 constexpr int kMinChunk = 128;      // tokens
 constexpr int kMaxChunk = 2048;
 constexpr int kTallChunk = 256;
+constexpr int kSmallLaunchTokens = 512;      // boxes up to this length stay whole in launches of less than a workgroup per CU
 constexpr int kLongHeadPerWaveChunk = 1024;   // tokens a wave walks alone (long boxes, a kv head per wave)
-constexpr int kTallChunkBusy = 768;          // tall chunk when the launch does not fit on the device at once
-constexpr int kResidentWgsPerCU = 3;
+// workgroups of the split kernel a CU holds at once: head_dim 128 -> 2 (registers and LDS of the 32-row tiles), 64 -> 3
+inline int resident_wgs_per_cu(int head_dim) { return head_dim == 128 ? 2 : 3; }
 
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
@@ -174,11 +175,12 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   auto round_unit = [&](int64_t c) { return std::max<int64_t>(unit, ceil_div64(c, unit) * unit); };
   const int64_t cap = (int64_t)kMaxChunkPages * page / unit * unit;  // page ids of a chunk sit in 2 VGPRs
   if (cap <= 0) return fail(PAT_ERR_INVALID, "page size too large for one workgroup");
-  int64_t work = 0, tall_work = 0;
+  int64_t work = 0;
   for (int i = 0; i < a->num_buckets; ++i) {
     const int64_t w = (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
-    if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w; else tall_work += w;
+    if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w;
   }
+  const int64_t resident = (int64_t)resident_wgs_per_cu(a->head_dim) * kNumCUs;
   int64_t chunk = tune.chunk_tokens, tall = tune.tall_chunk_tokens;
   const bool env_tall = tall > 0, env_chunk = chunk > 0;
   if (chunk <= 0) {
@@ -188,34 +190,34 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     chunk = std::max<int64_t>(kMinChunk, std::min<int64_t>(kMaxChunk, chunk));
   }
   if (tall <= 0) {
-    // at least kTallChunk; longer when the tall boxes alone would still fill the device
-    tall = ceil_div64(tall_work / (kTargetWgsPerCU * kNumCUs), 128) * 128;
+    // Tall boxes are cut only as far as it takes to have about three workgroups per eight CUs (with
+    // fewer, a tall workgroup's chain of 64-token super-steps is the launch's critical path:
+    // 2048 tokens of a lone box run ~45 us); beyond that every further piece only adds 16-32 KB of
+    // partial rows and a merge slot per row. Measured on the benchmark workloads: the shared
+    // 2048-token prefix of 64 requests (4 boxes x 8 kv heads) is fastest in 3-4 pieces, 16 boxes
+    // and more uncut.
+    int64_t tall_box_heads = 0, widest_tall = 0;
+    for (int i = 0; i < a->num_buckets; ++i)
+      if (row_tiles(a->buckets[i].mnw[0]) > 1 && a->buckets[i].num_boxes > 0) {
+        tall_box_heads += (int64_t)a->buckets[i].num_boxes * a->kv_heads;
+        widest_tall = std::max<int64_t>(widest_tall, (int64_t)a->buckets[i].max_blocks * page);
+      }
+    const int64_t pieces = tall_box_heads > 0 ? std::max<int64_t>(1, ceil_div64(3 * kNumCUs / 8, tall_box_heads)) : 1;
+    tall = ceil_div64(ceil_div64(widest_tall, pieces), 128) * 128;
     tall = std::max<int64_t>(kTallChunk, std::min<int64_t>(kMaxChunk, tall));
   }
-  if (!env_tall) {
-    // Does the launch fit on the device at once (3 workgroups per CU)? When it is well past that,
-    // workgroups start in launch order as others retire and the tall boxes are off the critical
-    // path: they then get at least 768 tokens per workgroup (fewer, longer workgroups: their
-    // 16..32 KB of partial rows each are the expensive part). Short boxes keep their size: with
-    // the launch tables ordered longest first, finer chunks no longer pack better.
-    int64_t n = 0, n_tall = 0;
-    for (int i = 0; i < a->num_buckets; ++i) {
-      const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
-      const bool is_tall = row_tiles(a->buckets[i].mnw[0]) > 1;
-      const int64_t c = is_tall ? round_unit(tall) : round_unit(chunk);
-      const int64_t wgs = (int64_t)a->buckets[i].num_boxes * std::max<int64_t>(1, ceil_div64(tok, c)) * a->kv_heads;
-      n += wgs;
-      if (is_tall) n_tall += wgs;
-    }
-    // (a handful of tall boxes stays finely cut: there the tall chain is the critical path)
-    if (2 * n > 3 * (int64_t)kResidentWgsPerCU * kNumCUs && n_tall >= kNumCUs)
-      tall = std::max<int64_t>(tall, kTallChunkBusy);
+  if (!env_tall && !env_chunk) {
     // Tall workgroups start first and stay for most of the launch. When they take more than a
     // third of the resident slots, the short boxes' chunk is sized for the slots that are left
     // (at least one per CU) instead of for two per CU: short workgroups that have to queue behind
     // the tall ones start late and make the tail.
-    else if (!env_chunk && n_tall > kNumCUs) {
-      const int64_t slots = std::max<int64_t>(kNumCUs, (int64_t)kResidentWgsPerCU * kNumCUs - n_tall);
+    int64_t n_tall = 0;
+    for (int i = 0; i < a->num_buckets; ++i)
+      if (row_tiles(a->buckets[i].mnw[0]) > 1)
+        n_tall += (int64_t)a->buckets[i].num_boxes *
+                  std::max<int64_t>(1, ceil_div64((int64_t)a->buckets[i].max_blocks * page, round_unit(tall))) * a->kv_heads;
+    if (n_tall > kNumCUs) {
+      const int64_t slots = std::max<int64_t>(kNumCUs, resident - n_tall);
       const int64_t c = std::min<int64_t>(kMaxChunk, ceil_div64(ceil_div64(work, slots), 128) * 128);
       chunk = std::max(chunk, c);
     }
@@ -233,8 +235,11 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
       if (a->buckets[i].num_boxes > 0) widest = std::max<int64_t>(widest, (int64_t)a->buckets[i].max_blocks * page);
     int64_t boxes = 0;
     for (int i = 0; i < a->num_buckets; ++i) boxes += a->buckets[i].num_boxes;
-    // (with fewer boxes than one per CU and kv head, cutting them is what fills the device)
-    if (widest > 0 && round_unit(widest) <= std::min<int64_t>(cap, kMaxChunk) && boxes * a->kv_heads >= kNumCUs) {
+    // (with fewer boxes than one per CU and kv head, cutting them is what fills the device - unless they are so
+    // short that a workgroup's four waves walk a whole box in a few steps each: then the second launch and its
+    // round trips cost more than the cuts save; 8 requests of 288 tokens, 8 kv heads: 7.6 -> 5 us)
+    if (widest > 0 && round_unit(widest) <= std::min<int64_t>(cap, kMaxChunk) &&
+        (boxes * a->kv_heads >= kNumCUs || widest <= kSmallLaunchTokens)) {
       chunk = std::max(chunk, widest);
       tall = std::max(tall, widest);
       single_slot = true;
@@ -264,7 +269,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     // start: the longest workgroup then sets when they are done. When they start in waves, the
     // remainders, which the chunk-major order launches last, make the shorter tail.
     const int64_t kind_wgs = row_tiles(a->buckets[i].mnw[0]) > 1 ? kind_tall_wgs : kind_short_wgs;
-    if (equalize == 1 || (equalize < 0 && kind_wgs <= (int64_t)kResidentWgsPerCU * kNumCUs))
+    if (equalize == 1 || (equalize < 0 && kind_wgs <= resident))
       c = std::min(c, round_unit(ceil_div64(tok, n)));
     g->bucket_chunk[i] = (int)c;
     g->bucket_chunks[i] = n;
@@ -279,7 +284,7 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   if (g->total_wgs >= 2 * kNumCUs && a->kv_heads % kWaves == 0) {
     // up to 256 tokens when the launch does not fit on the device at once, up to 128 when it
     // does (every workgroup is resident from the start and the longest chain sets the time)
-    const int64_t limit = head_per_wave_tokens(tune, g->total_wgs > (int64_t)kResidentWgsPerCU * kNumCUs);
+    const int64_t limit = head_per_wave_tokens(tune, g->total_wgs > resident);
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
       if (row_tiles(a->buckets[i].mnw[0]) == 1 && g->bucket_chunks[i] == 1 && tok <= limit) {
@@ -296,22 +301,35 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   // on its longest chains instead: c3 +11 %, c2 +37 %). pat_fwd_tuning.head_per_wave_long_wgs overrides
   // the number of such workgroups a bucket must have (0: always, tuning and tests).
   if (a->kv_heads % kWaves == 0) {
-    int64_t need = 2 * (int64_t)kResidentWgsPerCU * kNumCUs;
+    int64_t need = 2 * resident;
     bool forced = false;
     if (tune.head_per_wave_long_wgs >= 0) { need = tune.head_per_wave_long_wgs; forced = true; }
     bool changed = false;
+    int64_t tall_wgs = 0;
+    for (int i = 0; i < a->num_buckets; ++i)
+      if (row_tiles(a->buckets[i].mnw[0]) > 1) tall_wgs += (int64_t)a->buckets[i].num_boxes * g->bucket_chunks[i] * a->kv_heads;
     for (int i = 0; i < a->num_buckets; ++i) {
       const int64_t tok = (int64_t)a->buckets[i].max_blocks * page;
       if (row_tiles(a->buckets[i].mnw[0]) != 1 || g->bucket_heads_per_wg[i] != 1 || tok <= 256) continue;
       int64_t want = kLongHeadPerWaveChunk;
       if (tune.head_per_wave_long_tokens > 0) want = std::max<int64_t>(32, tune.head_per_wave_long_tokens);
+      // Boxes of up to 512 tokens whose 256-token pieces all find a place beside the tall workgroups
+      // (the private suffixes of a batch that shares one long prefix): a kv head per wave on those
+      // pieces - 8-step chains, a quarter of the workgroups of the steps-over-waves form and none
+      // of its LDS combines (64 requests over a 2048-token prefix: 30.4 -> 27.1 us per call). Not in
+      // small launches, where every wave of a workgroup is needed on one head: at least a workgroup
+      // per two CUs of this kind.
+      const int64_t piece_wgs = (int64_t)a->buckets[i].num_boxes * ceil_div64(tok, 256) * (a->kv_heads / kWaves);
+      const bool short_pieces = !forced && tune.head_per_wave_long_tokens <= 0 && tok <= 512 && !single_slot &&
+                                piece_wgs >= kNumCUs / 2 && piece_wgs <= std::max<int64_t>(kNumCUs, resident - tall_wgs);
+      if (short_pieces) want = 256;
       const int64_t n = ceil_div64(tok, std::min(round_unit(want), cap));
       const int64_t c = std::min(round_unit(ceil_div64(tok, n)), cap);   // n even pieces of the widest box
       if (n > kMaxChunksPerRank) continue;
       if (single_slot && n > 1) continue;   // (one chunk per box is worth as much, and keeps the launch single-slot)
       // an even bucket (caller's hint) has no stragglers: one such workgroup per CU is enough
       const int64_t need_i = (a->buckets[i].flags & PAT_BUCKET_EVEN) && !forced ? std::min<int64_t>(need, kNumCUs) : need;
-      if ((int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need_i) continue;
+      if (!short_pieces && (int64_t)a->buckets[i].num_boxes * n * (a->kv_heads / kWaves) < need_i) continue;
       g->bucket_chunk[i] = (int)c;
       g->bucket_chunks[i] = (int)n;
       g->bucket_heads_per_wg[i] = kWaves;

@@ -430,6 +430,17 @@ struct KernelInfo {
   // the whole plan in one int32 buffer (pinned on the host when a GPU is there)
   std::optional<at::Tensor> flat;
   pat_flat_plan layout;
+  // Small batches of short requests (see whole_sequences_pay): what the tree form launches there is one
+  // work item per request over its own block row - a single kernel that writes `out`, where the
+  // prefix-aware plan needs a second one to merge two or three partial results per request. Its
+  // tables sit behind the plan in the same buffer: [batch] request ids, ones, zeros, lengths, then
+  // the block rows [batch, ws_width].
+  bool whole_seqs = false;
+  int64_t ws_offset = 0;
+  int ws_batch = 0, ws_width = 0, ws_tile = 16;
+  TensorList ws_q_table, ws_block_table, ws_num_seqs, ws_rank, ws_kv;
+  std::vector<std::vector<int>> ws_mnw;
+  at::Tensor ws_num_split;
   std::unordered_map<std::string, std::shared_ptr<Prepared>> cache;
   RecordStore records;
 
@@ -453,8 +464,10 @@ struct KernelInfo {
 
   void clear_tables() {
     for (TensorList* l : {&q_tables, &block_tables, &num_seqs, &ranks, &kvs, &slot_tables, &l_q_tables,
-                          &l_block_tables, &l_num_seqs, &l_ranks, &l_kvs, &l_slot_tables, &launch_order})
+                          &l_block_tables, &l_num_seqs, &l_ranks, &l_kvs, &l_slot_tables, &launch_order,
+                          &ws_q_table, &ws_block_table, &ws_num_seqs, &ws_rank, &ws_kv})
       l->clear();
+    ws_mnw.clear();
     mnws.clear(); l_mnws.clear(); l_flags.clear(); launch_parts.clear();
     cache.clear();
     records = RecordStore();
@@ -493,6 +506,16 @@ struct KernelInfo {
       launch_parts[(size_t)f.parent].push_back({i, f.first, f.first + f.num_boxes});
     }
     has_launch = true;
+    if (whole_seqs) {
+      const int64_t b = ws_batch;
+      ws_q_table.push_back(mat(ws_offset, b, 1));
+      ws_num_seqs.push_back(vec(ws_offset + b, b));
+      ws_num_split = vec(ws_offset + b, b);          // (ones as well: every request is one work item)
+      ws_rank.push_back(vec(ws_offset + 2 * b, b));
+      ws_kv.push_back(vec(ws_offset + 3 * b, b));
+      ws_block_table.push_back(mat(ws_offset + 4 * b, b, ws_width));
+      ws_mnw.push_back({ws_tile, 128, 1});
+    }
   }
 
   // Copies every plan tensor to `device`: one copy of the one buffer, asynchronous from pinned memory
@@ -528,6 +551,17 @@ struct KernelInfo {
     return d;
   }
 
+  // The tables of the one-work-item-per-request launch, or None when the plan is launched as planned.
+  py::object whole_sequence_tables() const {
+    if (!whole_seqs) return py::none();
+    py::dict d;
+    d["q_tables"] = ws_q_table; d["block_tables"] = ws_block_table; d["num_seqs_per_CTAs"] = ws_num_seqs;
+    d["CTA_ranks"] = ws_rank; d["kv_in_CTAs"] = ws_kv; d["MNWs"] = ws_mnw;
+    d["num_split_per_seq"] = ws_num_split; d["max_split_per_seq"] = 1; d["max_seqs_in_CTA"] = 1;
+    d["max_blocks_in_CTA"] = ws_width;
+    return d;
+  }
+
   // For the boxes of scheduler bucket b, in scheduler order: (launch bucket, row in it).
   std::pair<at::Tensor, at::Tensor> launch_position(int b) const {
     require(b >= 0 && (size_t)b < launch_order.size(), "bucket index out of range");
@@ -555,8 +589,23 @@ struct TreeHandle {
   ~TreeHandle() { if (h) pat_tree_destroy(h); }
 };
 
+// Is a batch better served by one work item per request than by its prefix-aware plan? Yes when the
+// whole launch is a few microseconds of latency anyway: every request short enough for one workgroup
+// to walk in a few steps per wave, at most two workgroups per CU, and so little KV in total that
+// re-reading shared pages (from L2) costs less than the merge kernel's launch and round trips.
+bool whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page) {
+  if (lens.empty() || kv_heads <= 0) return false;
+  int64_t total = 0, longest = 0;
+  for (int32_t n : lens) { total += n; longest = std::max<int64_t>(longest, n); }
+  const int64_t bytes = total * kv_heads * 128 * 2 * 2;   // (at head_dim 128; the planner does not know it)
+  return longest > 0 && longest <= 512 && (int64_t)lens.size() * kv_heads <= 512 && bytes <= (int64_t)16 << 20 &&
+         page > 0;
+}
+
 struct PrefixTreeCPP {
   int block_size;
+  std::vector<int32_t> batch_lens;   // the batch as build_radix_tree got it
+  at::Tensor batch_table;
   std::shared_ptr<TreeHandle> native = std::make_shared<TreeHandle>();
   std::shared_ptr<KernelInfo> info = std::make_shared<KernelInfo>();
 
@@ -585,6 +634,8 @@ struct PrefixTreeCPP {
       throw std::runtime_error("seq_lens must be a List[int] or a CPU Int32 Tensor");
     }
     require(n_lens == table.size(0), "Seq lens list mismatch");
+    batch_lens.assign(lens, lens + n_lens);
+    batch_table = table;
     int rc;
     {
       py::gil_scoped_release release;   // the tree is built without the GIL (csrc/bindings.cpp:124)
@@ -617,13 +668,37 @@ struct PrefixTreeCPP {
     check(rc);
     c10::InferenceMode plain(false);   // plan tensors keep their version counters (see KernelInfo::to_gpu)
     if (rc_flat == PAT_OK) {
-      const int64_t total = std::max<int64_t>(fresh->layout.total, 1);
+      int64_t total = std::max<int64_t>(fresh->layout.total, 1);
+      const int64_t nb = (int64_t)batch_lens.size();
+      if (hratio >= 1 && hratio <= 16 && fresh->layout.batch == nb && batch_table.defined() && batch_table.size(0) == nb &&
+          whole_sequences_pay(batch_lens, kv_head, block_size)) {
+        int64_t longest = 0;
+        for (int32_t n : batch_lens) longest = std::max<int64_t>(longest, n);
+        fresh->whole_seqs = true;
+        fresh->ws_batch = (int)nb;
+        // (8 spare columns: room for in-place growth between decode steps)
+        fresh->ws_width = (int)std::min<int64_t>(batch_table.size(1), (longest + block_size - 1) / block_size + 8);
+        fresh->ws_tile = 16;
+        fresh->ws_offset = total;
+        total += 4 * nb + nb * fresh->ws_width;
+      }
       host = at::empty({total}, at::TensorOptions().dtype(at::kInt).pinned_memory(at::hasHIP() || at::hasCUDA()));
       {
         py::gil_scoped_release release;
         rc = pat_tree_flat_plan(native->h, &fresh->layout, host.data_ptr<int32_t>(), host.numel());
       }
       check(rc);
+      if (fresh->whole_seqs) {
+        const int64_t nb = fresh->ws_batch, w = fresh->ws_width;
+        int32_t* d = host.data_ptr<int32_t>() + fresh->ws_offset;
+        const int32_t* src = batch_table.data_ptr<int32_t>();
+        const int64_t src_w = batch_table.size(1);
+        for (int64_t i = 0; i < nb; ++i) {
+          d[i] = (int32_t)i; d[nb + i] = 1; d[2 * nb + i] = 0; d[3 * nb + i] = batch_lens[(size_t)i];
+          const int64_t used = ((int64_t)batch_lens[(size_t)i] + block_size - 1) / block_size;
+          for (int64_t j = 0; j < w; ++j) d[4 * nb + i * w + j] = j < used ? src[i * src_w + j] : 0;
+        }
+      }
       fresh->flat = host;
       fresh->max_split = fresh->layout.max_split_per_seq;
       fresh->max_boxes = fresh->layout.max_boxes_per_seq;
@@ -771,8 +846,15 @@ void fwd_tree(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, Pre
                   l ? &info.l_slot_tables : &info.slot_tables, l ? &info.l_mnws : &info.mnws,
                   l ? &info.l_flags : &no_flags};
     require(!pt.mnw->empty(), "the tree has no plan: call pack_schedule and kernel_info.to_gpu first");
-    L = prepare(q, k, v, info.num_boxes_per_seq, pt, info.max_boxes, info.max_seqs, info.max_blocks, scale, out, lse,
-                info.records, version);
+    if (info.whole_seqs && !info.ws_q_table.empty()) {
+      // a small batch of short requests: one work item per request, one kernel (see KernelInfo::whole_seqs)
+      PlanTables ws{&info.ws_q_table, &info.ws_block_table, &info.ws_num_seqs, &info.ws_rank, &info.ws_kv, nullptr,
+                    &info.ws_mnw, &no_flags};
+      L = prepare(q, k, v, info.ws_num_split, ws, 1, 1, info.ws_width, scale, out, lse, info.records, version);
+    } else {
+      L = prepare(q, k, v, info.num_boxes_per_seq, pt, info.max_boxes, info.max_seqs, info.max_blocks, scale, out, lse,
+                  info.records, version);
+    }
     if (info.cache.size() >= 256) info.cache.clear();
     info.cache[key.bytes] = L;
   }
@@ -851,6 +933,10 @@ PYBIND11_MODULE(_prefix_attn, m) {
       .def("launch_tables", &KernelInfo::launch_tables,
            "The per-bucket tables as the kernels get them (boxes longest first, a bucket with a wide head split "
            "in two) with their tile labels under \"MNWs\" and hints under \"flags\".")
+      .def("whole_sequence_tables", &KernelInfo::whole_sequence_tables,
+           "Small batches of short requests are launched as one work item per request (a single kernel that "
+           "writes `out`): the tables of that launch, with its num_split_per_seq / max_* values, or None when "
+           "the plan is launched as planned.")
       .def("launch_position", &KernelInfo::launch_position, py::arg("bucket"),
            "For the boxes of a scheduler bucket, in scheduler order: (launch bucket, row in it) as two int64 tensors.")
       .def_property_readonly("_flat", [](const KernelInfo& ki) -> py::object {

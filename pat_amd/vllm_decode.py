@@ -146,8 +146,23 @@ class DecodePlan:
                     if (np.asarray(cols)[which] >= tables[t].shape[1]).any():
                         self._replan(table_cpu)
                         return False
+        # a small batch that is launched as one work item per request (KernelInfo.whole_sequence_tables):
+        # those tables grow too; a request that outgrows its block row, or the form, means a fresh plan
+        whole = info.whole_sequence_tables()
+        if whole is not None:
+            width = whole["block_tables"][0].shape[1]
+            if any(n_old % bs == 0 and n_old // bs >= width for n_old in old) or max(self.seq_lens) > 512:
+                self._replan(table_cpu)
+                return False
         self._tail_kv += 1
         device = info.num_split_per_seq.device
+        if whole is not None:
+            whole["kv_in_CTAs"][0].add_(1)
+            crossed = [s for s, n_old in enumerate(old) if n_old % bs == 0]
+            if crossed:
+                flat = torch.as_tensor([s * width + old[s] // bs for s in crossed], device=device)
+                ids = torch.as_tensor([int(table_cpu[s, old[s] // bs]) for s in crossed], dtype=torch.int32, device=device)
+                whole["block_tables"][0].view(-1).index_copy_(0, flat, ids)
         for kvs, tables, place in targets:
             for b in range(len(info.MNWs)):
                 grown = self._tails[self._tails[:, 0] == b, 1]

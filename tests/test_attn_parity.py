@@ -1070,3 +1070,35 @@ def test_first_call_under_capture_then_eager():
     graph.replay()
     torch.cuda.synchronize()
     assert (out_graph.float().cpu() - ref_out.float()).abs().max().item() <= TOL[w.dtype]
+
+
+def test_small_batch_is_launched_as_whole_sequences():
+    # 8 requests of 288 tokens: the tree form launches one work item per request - a single kernel
+    # that writes `out` (no workspace, no merge) - and still equals the oracle; the plan tables stay
+    # what the scheduler made
+    print("[case] small batch (c1): one work item per request", flush=True)
+    dev = _device()
+    w = workloads.make("c1", seed=8)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    whole = info.whole_sequence_tables()
+    assert whole is not None and whole["max_split_per_seq"] == 1
+    assert whole["kv_in_CTAs"][0].tolist() == list(w.seq_lens)
+    assert info.max_split_per_seq >= 2            # the scheduler's plan: shared prefix boxes and a private one each
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    assert info._launch_workspace_bytes == [0]
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("whole sequences", out, lse, ref_out, ref_lse, w.dtype)
+    # a batch of the same shape with longer requests is launched as planned
+    big = workloads.make("c2", seed=8)
+    t2 = PrefixTreeCPP(big.page_size)
+    t2.build_radix_tree(big.seq_lens, big.padded_table())
+    t2.pack_schedule(None, big.heads // big.kv_heads, big.kv_heads)
+    assert t2.kernel_info.whole_sequence_tables() is None

@@ -112,10 +112,13 @@ def test_geometry_and_workspace_are_consistent():
     g = _lib.FwdGeometry()
     assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
     assert g.chunk_tokens % 32 == 0 and g.tall_chunk_tokens % 32 == 0
-    per_box = [-(-128 * 16 // g.tall_chunk_tokens), -(-32 * 16 // g.chunk_tokens)]
+    # 4 tall boxes x 8 kv heads are cut until there are about three workgroups per eight CUs: 3 pieces;
+    # the 64 boxes of up to 512 tokens run a kv head per wave on 256-token pieces (2 per box, 2 head groups)
+    per_box = [3, 2]
+    assert -(-128 * 16 // g.tall_chunk_tokens) == per_box[0]
     assert g.chunks_per_rank == max(per_box)
     assert g.num_slots == g.chunks_per_rank * 2
-    assert g.num_workgroups == 8 * (4 * per_box[0] + 64 * per_box[1])
+    assert g.num_workgroups == 8 * 4 * per_box[0] + 64 * per_box[1] * (8 // 4)
     need = C.c_size_t()
     assert lib.pat_fwd_workspace_bytes(C.byref(a), C.byref(need)) == 0
     rows = 64 * 32 * g.num_slots

@@ -164,6 +164,12 @@ def test_advance_step_keeps_the_plan_right_on_cpu(case):
                     assert torch.equal(launch["kv_in_CTAs"][lb], info.kv_in_CTAs[b][order[lo:hi]])
                     assert torch.equal(launch["block_tables"][lb], info.block_tables[b][order[lo:hi]][:, :lw])
                     assert (launch["kv_in_CTAs"][lb][:-1] >= launch["kv_in_CTAs"][lb][1:] - step).all()
+            whole = info.whole_sequence_tables()    # small batches are launched a work item per request
+            assert (whole is not None) == (case == "c1")
+            if whole is not None:
+                assert whole["kv_in_CTAs"][0].tolist() == lens and whole["q_tables"][0][:, 0].tolist() == list(range(w.batch))
+                for i, r in enumerate(rows):
+                    assert whole["block_tables"][0][i, :len(r)].tolist() == r
             out, lse = ao.run_plan_ref(listed, q, k, v)
             ref, ref_lse = ao.paged_attention_ref(q, k, v, rows, lens)
             assert (out - ref).abs().max().item() < 1e-5, step
@@ -173,10 +179,12 @@ def test_advance_step_keeps_the_plan_right_on_cpu(case):
 
 
 @pytest.mark.gpu
-def test_advance_step_on_gpu():
-    print("[case] vLLM multi-step advance c2", flush=True)
+@pytest.mark.parametrize("name", ["c2", "c1"])
+def test_advance_step_on_gpu(name):
+    # (c1: a batch small enough to be launched as one work item per request; those tables grow too)
+    print(f"[case] vLLM multi-step advance {name}", flush=True)
     dev = torch.device("cuda:0")
-    w = workloads.make("c2", seed=6)
+    w = workloads.make(name, seed=6)
     steps = 18
     spare = list(range(w.num_blocks, w.num_blocks + 2 * w.batch))
     width = w.padded_table().shape[1] + 2
@@ -200,4 +208,4 @@ def test_advance_step_on_gpu():
             ref, _ = ao.paged_attention_ref(q, k, v, rows, lens)
             err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
             print(f"[parity] advance step {step}: max|out - ref| = {err:.3e} (replans {plan.replans})", flush=True)
-            assert err <= 1.6e-2
+            assert err <= (1.6e-2 if w.dtype == torch.bfloat16 else 2e-3)
