@@ -357,7 +357,11 @@ int pat_fwd_launch(const pat_fwd_args* args, void* hip_stream);
  * space than the array holds fails with PAT_ERR_WORKSPACE and enqueues nothing. Every call on a GPU
  * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls
  * on one stream are ordered and safe. Nothing in the array has to be cleared between calls: every
- * slot a call reads it writes first (slots filed as described at pat_fwd_bucket.q_slot). */
+ * slot a call reads it writes first (slots filed as described at pat_fwd_bucket.q_slot).
+ * The first call on each device looks up the array's device address (hipGetSymbolAddress, which may
+ * load the code object) and therefore must not be made while `hip_stream` is capturing: it fails with
+ * PAT_ERR_INVALID there and enqueues nothing. Make one call on the device before the capture; later
+ * calls, captured or not, only enqueue kernels. */
 int pat_fwd_launch_static(const pat_fwd_args* args, void* hip_stream);
 size_t pat_fwd_static_scratch_bytes(void);
 

@@ -753,6 +753,14 @@ int pat_fwd_launch_static(const pat_fwd_args* args, void* hip_stream) {
   {
     std::lock_guard<std::mutex> lock(mutex);
     if (device_ptr[dev] == nullptr) {
+      // the lookup may load the code object (a device allocation of the runtime's own), which a
+      // stream capture in progress does not allow: the first call on a device has to come before it
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      if (const hipError_t e = hipStreamIsCapturing(static_cast<hipStream_t>(hip_stream), &capturing); e != hipSuccess)
+        return hip_fail(e, "hipStreamIsCapturing");
+      if (capturing != hipStreamCaptureStatusNone)
+        return fail(PAT_ERR_INVALID, "pat_fwd_launch_static: the first call on a device looks up the scratch array and "
+                                     "cannot run under stream capture; call it once on this device before capturing");
       void* found = nullptr;
       if (const hipError_t e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)); e != hipSuccess)
         return hip_fail(e, "hipGetSymbolAddress(scratch)");

@@ -18,6 +18,7 @@
 
 #include <cstring>
 #include <memory>
+#include <atomic>
 #include <mutex>
 #include <optional>
 #include <string>
@@ -92,6 +93,7 @@ struct Prepared {
 // rounded up to multiples of 8.
 std::mutex g_tune_mutex;
 std::unordered_map<std::string, pat_fwd_tuning> g_tuned;
+std::atomic<int64_t> g_tuning_runs{0};   // measurements made since the module was loaded
 // Opt-in (PAT_AUTOTUNE=1 or set_autotune(True)): the measurement synchronises the stream and runs
 // the launch some fifty times, which a serving loop must not meet unasked; the automatic geometry
 // (sizes only) is the default.
@@ -146,6 +148,7 @@ void tune(Prepared& L, const c10::Device& dev) {
     evict = it->second;
   }
   pat_fwd_tuning best;
+  g_tuning_runs.fetch_add(1);
   const int rc = pat_fwd_autotune(&L.args, stream, 8, evict.data_ptr(), (size_t)evict.numel(), &best, nullptr, nullptr);
   L.args.workspace = nullptr; L.args.workspace_bytes = 0;
   check(rc);
@@ -999,6 +1002,8 @@ PYBIND11_MODULE(_prefix_attn, m) {
         "unless switched on here or with PAT_AUTOTUNE=1. The measurement runs the launch some fifty times on the "
         "current stream and synchronises it, once per shape.");
   m.def("get_autotune", [] { return g_autotune; });
+  m.def("autotune_runs", [] { return g_tuning_runs.load(); },
+        "Number of geometry measurements made since the module was loaded (0 unless tuning was switched on).");
   m.def("clear_autotune_cache", [] { std::lock_guard<std::mutex> lock(g_tune_mutex); g_tuned.clear(); });
   m.def("paged_decode_baseline", &paged_decode_baseline, py::arg("q"), py::arg("k_cache_paged"),
         py::arg("v_cache_paged"), py::arg("block_table"), py::arg("seq_lens"), py::arg("softmax_scale"), py::arg("out"),

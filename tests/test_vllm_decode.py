@@ -209,3 +209,76 @@ def test_advance_step_on_gpu(name):
             err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
             print(f"[parity] advance step {step}: max|out - ref| = {err:.3e} (replans {plan.replans})", flush=True)
             assert err <= (1.6e-2 if w.dtype == torch.bfloat16 else 2e-3)
+
+
+@pytest.mark.gpu
+def test_fifty_replanned_decode_steps_with_requests_leaving_and_joining():
+    """A serving loop on the headline batch: every step each request grows by a token, every fifth
+    step one request finishes and a new one (same shared prefix, fresh suffix) takes its row, and
+    the plan is built afresh from the step's metadata. Default settings make no tuning run at all;
+    with tuning switched on the whole loop makes one per distinct plan shape it meets (a handful: the
+    shape key rounds box counts and widths up to multiples of 8), never one per step.
+    Parity against the dense reference on the step's own tables at several steps of both loops."""
+    from pat_amd import _prefix_attn as ext
+    print("[case] 50 re-planned decode steps of c2, requests leaving and joining", flush=True)
+    dev = torch.device("cuda:0")
+    w = workloads.make("c2", seed=8)
+    steps, page = 50, w.page_size
+    shared = min(len(r) for r in w.rows)
+    prefix = None
+    for depth in range(shared):                      # pages every request starts with
+        if len({r[depth] for r in w.rows}) != 1:
+            break
+        prefix = depth + 1
+    assert prefix and prefix * page >= 2048
+    spare_blocks = 4 * w.batch + 12 * 40
+    gen = torch.Generator().manual_seed(5)
+    q = torch.randn(w.batch, 1, w.heads, w.head_dim, generator=gen).to(w.dtype)
+    k = torch.randn(w.num_blocks + spare_blocks, page, w.kv_heads, w.head_dim, generator=gen).to(w.dtype)
+    v = torch.randn(w.num_blocks + spare_blocks, page, w.kv_heads, w.head_dim, generator=gen).to(w.dtype)
+    kv_cache = torch.stack([k, v]).to(dev)
+    query = q.squeeze(1).to(dev)
+    output = torch.empty_like(query)
+    width = w.padded_table().shape[1] + 8
+
+    def serve(tuning_on):
+        rows, lens = [list(r) for r in w.rows], list(w.seq_lens)
+        spare = iter(range(w.num_blocks, w.num_blocks + spare_blocks))
+        ext.set_autotune(tuning_on)
+        ext.clear_autotune_cache()
+        before = ext.autotune_runs()
+        worst = 0.0
+        try:
+            for step in range(1, steps + 1):
+                for i in range(w.batch):                       # one more token each
+                    if lens[i] % page == 0:
+                        rows[i].append(next(spare))
+                    lens[i] += 1
+                if step % 5 == 0:                              # one leaves, one joins on its row
+                    i = (7 * step) % w.batch
+                    fresh = 64 + (37 * step) % 448
+                    rows[i] = rows[i][:prefix] + [next(spare) for _ in range(-(-fresh // page))]
+                    lens[i] = prefix * page + fresh
+                table = _table(rows, width)
+                meta = SimpleNamespace(num_prefills=0, num_decode_tokens=w.batch, seq_lens=list(lens),
+                                       block_tables=table.to(dev), block_tables_cpu=table, block_size=page,
+                                       nheads=w.heads, nheads_kv=w.kv_heads, max_decode_query_len=1)
+                plan = DecodePlan.from_metadata(meta)
+                decode_attention(query, kv_cache, plan, 1.0 / math.sqrt(w.head_dim), output)
+                if step in (1, 5, 26, 50):
+                    torch.cuda.synchronize()
+                    ref, _ = ao.paged_attention_ref(q, k, v, rows, lens)
+                    err = (output.unsqueeze(1).float().cpu() - ref.float()).abs().max().item()
+                    worst = max(worst, err)
+                    assert err <= 1.6e-2, (step, err)
+            torch.cuda.synchronize()
+        finally:
+            ext.set_autotune(False)
+        return ext.autotune_runs() - before, worst
+
+    runs, worst = serve(False)
+    print(f"[parity] default settings: {runs} tuning runs, max|out - ref| = {worst:.3e}", flush=True)
+    assert runs == 0
+    runs, worst = serve(True)
+    print(f"[parity] tuning switched on: {runs} tuning runs over {steps} plans, max|out - ref| = {worst:.3e}", flush=True)
+    assert runs <= 4
