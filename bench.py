@@ -43,22 +43,21 @@ INFINITY_CACHE_BYTES = 256 << 20
 
 def measured_traffic_bytes(workload: str, seed: int, workgroups: int):
     """HBM bytes per split-kernel launch as rocprofv3 measured them (--pmc FETCH_SIZE + WRITE_SIZE, each
-    scaled by the same counter's reading for a 1 GiB copy kernel), from the marker lines of
-    profiles/pat_split_kernel_<workload>.md (one per launch geometry that was measured). None when
+    scaled by the same counter's reading for a 1 GiB copy kernel), from the marker lines of the
+    summaries under profiles/ (one per workload and launch geometry that was measured). None when
     there is no such measurement for this workload, seed and number of workgroups, or when the
     kernel sources have changed since it was taken."""
+    import glob
     import hashlib
     import re
-    path = os.path.join(ROOT, "profiles", f"pat_split_kernel_{workload}.md")
-    if not os.path.exists(path):
-        return None
     h = hashlib.sha256()
     for rel in ("pat_amd/csrc/hip/pat_split.hip", "pat_amd/csrc/hip/fwd_params.hpp", "pat_amd/csrc/capi_fwd.hip"):
         h.update(open(os.path.join(ROOT, rel), "rb").read())
-    for m in re.finditer(r"bench-marker: workload=(\S+) seed=(\d+) workgroups=(\d+) traffic_bytes=(\d+) "
-                         r"kernel_sources_sha256=([0-9a-f]+)", open(path).read()):
-        if m.group(1) == workload and int(m.group(2)) == seed and int(m.group(3)) == workgroups and h.hexdigest() == m.group(5):
-            return int(m.group(4))
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "pat_split_kernel_*.md"))):
+        for m in re.finditer(r"bench-marker: workload=(\S+) seed=(\d+) workgroups=(\d+) traffic_bytes=(\d+) "
+                             r"kernel_sources_sha256=([0-9a-f]+)", open(path).read()):
+            if m.group(1) == workload and int(m.group(2)) == seed and int(m.group(3)) == workgroups and h.hexdigest() == m.group(5):
+                return int(m.group(4))
     return None
 
 WORKLOAD_TEXT = {

@@ -178,6 +178,9 @@ def load() -> C.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m pat_amd.build` "
             "(hipcc, --offload-arch=gfx950). pat_amd has no CPU fallback.")
+    # torch ships a HIP runtime of its own; loading it first lets the dynamic loader hand that same
+    # runtime to this library (one runtime per process, whatever the import order of the caller)
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SYMBOLS.items():
         fn = getattr(lib, name)
