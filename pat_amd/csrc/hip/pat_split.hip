@@ -462,12 +462,17 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
 
     // One 32-token step of online-softmax attention for this wave's 32 rows against a stage.
     auto attend32 = [&](const PAT_LDS char* stage, int t0) {
+      // every K operand of the step is requested before the first MFMA waits for one (left alone, the
+      // compiler reads each operand right ahead of its use and exposes the LDS latency KK2 times)
+      vec8 kop[KK2];
+#pragma unroll
+      for (int kk = 0; kk < KK2; ++kk) kop[kk] = *(const PAT_LDS vec8*)(stage + k_rd + kk * 32);
+      __builtin_amdgcn_sched_barrier(0);
       f32x16 s;
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-      for (int kk = 0; kk < KK2; ++kk)
-        s = E::mfma32(*(const PAT_LDS vec8*)(stage + k_rd + kk * 32), q2[kk], s);
+      for (int kk = 0; kk < KK2; ++kk) s = E::mfma32(kop[kk], q2[kk], s);
       // The rows' reference maxima move only when some row's maximum has left a window of kLazy
       // (base-2 exponent units) above its reference: probabilities then reach 2^kLazy at most, which
       // fp32 sums and 16-bit P hold as well as values below 1, and the accumulator is rescaled a few
