@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PAT_ABI_VERSION 3
+#define PAT_ABI_VERSION 4
 
 /* ---- status codes ------------------------------------------------------- */
 #define PAT_OK 0
@@ -142,6 +142,24 @@ int pat_tree_build_rows(pat_tree* tree, const int32_t* seq_lens,
                         const int32_t* flat_blocks, const int64_t* row_offsets,
                         int32_t num_seqs);
 
+/* Edits of a built tree between decode steps. No counterpart in the reference, which builds a new
+ * tree from the whole batch for every step (plugin/vllm/attention/backends/prefix_attn.py:330-338,
+ * 377-448). Sequence ids are batch rows:
+ *   pat_tree_append  adds a row behind the last one (its id = pat_tree_num_seqs before the call);
+ *   pat_tree_remove  deletes row `seq`; the rows behind it move up by one;
+ *   pat_tree_grow    lengthens row `seq` to new_len tokens; more_blocks are the blocks it gained.
+ * After any of them the tree, and every plan packed from it, is what pat_tree_build_rows gives for
+ * the edited batch (same nodes, child order, sequence lists, token counts; split counters of a
+ * fresh tree), provided that every block two rows share is full for both - what a paged KV cache
+ * with prefix sharing guarantees. pat_tree_grow returns PAT_ERR_VALUE and leaves the tree as it was
+ * when only a fresh build can know the new shape (the row grew inside a shared block, or into blocks
+ * another row holds): build the tree again then. */
+int pat_tree_append(pat_tree* tree, int32_t seq_len, const int32_t* blocks, int32_t num_blocks);
+int pat_tree_remove(pat_tree* tree, int32_t seq);
+int pat_tree_grow(pat_tree* tree, int32_t seq, int32_t new_len, const int32_t* more_blocks,
+                  int32_t num_more);
+int pat_tree_num_seqs(const pat_tree* tree);
+
 /* PrefixTree.pack_schedule(MNWs, HRatio, kvHead, use_compute_model)
  *                                             prefix_attn/prefix_tree.py:548-616
  * mnws: n_mnws triples [M, N, W] or NULL (n_mnws 0) for the default 11 buckets.
@@ -207,6 +225,7 @@ int pat_tree_flat_plan(const pat_tree* tree, pat_flat_plan* layout, int32_t* dst
 /* Borrow the plan built by the last pack / naive_schedule call. */
 int pat_tree_plan(const pat_tree* tree, pat_plan_view* out);
 
+/* Node slots of the tree (slots given up by pat_tree_remove included: their parent is -2). */
 int pat_tree_num_nodes(const pat_tree* tree);
 int pat_tree_node(const pat_tree* tree, int32_t node, pat_node_view* out);
 

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpat_amd.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 PAT_OK = 0
 PAT_ERR_INVALID = -1
@@ -144,6 +144,10 @@ SYMBOLS = {
     "pat_tree_plan": (C.c_int, [C.c_void_p, C.POINTER(PlanView)]),
     "pat_tree_flat_plan": (C.c_int, [C.c_void_p, C.POINTER(FlatPlan), C.c_void_p, C.c_int64]),
     "pat_tree_num_nodes": (C.c_int, [C.c_void_p]),
+    "pat_tree_append": (C.c_int, [C.c_void_p, C.c_int32, i32p, C.c_int32]),
+    "pat_tree_remove": (C.c_int, [C.c_void_p, C.c_int32]),
+    "pat_tree_grow": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, i32p, C.c_int32]),
+    "pat_tree_num_seqs": (C.c_int, [C.c_void_p]),
     "pat_tree_node": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(NodeView)]),
     "pat_fwd_validate": (C.c_int, [C.POINTER(FwdArgs)]),
     "pat_fwd_workspace_bytes": (C.c_int, [C.POINTER(FwdArgs), C.POINTER(C.c_size_t)]),

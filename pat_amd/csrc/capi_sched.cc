@@ -102,6 +102,29 @@ int pat_tree_build(pat_tree* tree, const int32_t* seq_lens, const int32_t* table
   return pat_tree_build_rows(tree, seq_lens, flat.data(), offsets.data(), num_seqs);
 }
 
+int pat_tree_append(pat_tree* tree, int32_t seq_len, const int32_t* blocks, int32_t num_blocks) {
+  if (tree == nullptr) return pat::fail(PAT_ERR_INVALID, "tree is NULL");
+  if (seq_len < 0 || num_blocks < 0) return pat::fail(PAT_ERR_INVALID, "seq_len / num_blocks must be >= 0");
+  if (num_blocks > 0 && blocks == nullptr) return pat::fail(PAT_ERR_INVALID, "blocks is NULL");
+  return guarded([&] { tree->planner->append(seq_len, blocks, num_blocks); });
+}
+
+int pat_tree_remove(pat_tree* tree, int32_t seq) {
+  if (tree == nullptr) return pat::fail(PAT_ERR_INVALID, "tree is NULL");
+  return guarded([&] { tree->planner->remove(seq); });
+}
+
+int pat_tree_grow(pat_tree* tree, int32_t seq, int32_t new_len, const int32_t* more_blocks, int32_t num_more) {
+  if (tree == nullptr) return pat::fail(PAT_ERR_INVALID, "tree is NULL");
+  if (num_more > 0 && more_blocks == nullptr) return pat::fail(PAT_ERR_INVALID, "more_blocks is NULL");
+  return guarded([&] { tree->planner->grow(seq, new_len, more_blocks, num_more); });
+}
+
+int pat_tree_num_seqs(const pat_tree* tree) {
+  if (tree == nullptr) return pat::fail(PAT_ERR_INVALID, "tree is NULL");
+  return tree->planner->num_seqs();
+}
+
 int pat_tree_pack(pat_tree* tree, const int32_t* mnws, int32_t n_mnws, int32_t hratio,
                   int32_t kv_heads, int32_t use_compute_model, const pat_sched_opts* opts) {
   if (tree == nullptr) return pat::fail(PAT_ERR_INVALID, "tree is NULL");

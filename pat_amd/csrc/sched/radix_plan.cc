@@ -76,6 +76,12 @@ int RadixPlanner::add_node(int parent, int num_seqs, int num_tokens, std::vector
   n.num_tokens = num_tokens;
   n.seq_ids = std::move(seq_ids);
   n.blocks = std::move(blocks);
+  if (!free_nodes_.empty()) {
+    const int at = free_nodes_.back();
+    free_nodes_.pop_back();
+    nodes_[(size_t)at] = std::move(n);
+    return at;
+  }
   nodes_.push_back(std::move(n));
   return (int)nodes_.size() - 1;
 }
@@ -132,7 +138,136 @@ void RadixPlanner::build(const int32_t* seq_lens, const int32_t* flat_blocks,
     const int64_t b = row_offsets[i], e = row_offsets[i + 1];
     insert(i, seq_lens[i], flat_blocks + b, (int)(e - b));
   }
+  seq_len_.assign(seq_lens, seq_lens + num_seqs);
   split_per_seq_.assign((size_t)num_seqs, 0);
+}
+
+// ---- edits of a built tree ---------------------------------------------------------------------
+// The reference builds a new tree for every decode step
+// (plugin/vllm/attention/backends/prefix_attn.py:330-338); these keep one tree in step with the batch.
+// What makes the result equal to a fresh build: build() inserts rows in order, so a node's sequence
+// list is ascending, and the children of a node stand in the order of their smallest sequence id
+// (a child is created by the first row that needs it, and a cut keeps the cut child's place).
+
+std::vector<int> RadixPlanner::path_of(int seq) const {
+  std::vector<int> path;
+  int at = 0;
+  for (;;) {
+    int next = -1;
+    for (int child : nodes_[(size_t)at].child_ids) {
+      const auto& ids = nodes_[(size_t)child].seq_ids;
+      if (std::binary_search(ids.begin(), ids.end(), (int32_t)seq)) { next = child; break; }
+    }
+    if (next < 0) return path;
+    path.push_back(next);
+    at = next;
+  }
+}
+
+void RadixPlanner::release_node(int node) {
+  nodes_[(size_t)node] = RadixNode();
+  nodes_[(size_t)node].parent = -2;   // not part of the tree
+  nodes_[(size_t)node].num_seqs = 0;
+  free_nodes_.push_back(node);
+}
+
+void RadixPlanner::sort_children(int node) {
+  RadixNode& n = nodes_[(size_t)node];
+  std::vector<size_t> order(n.child_ids.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+  std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) {
+    return nodes_[(size_t)n.child_ids[a]].seq_ids.front() < nodes_[(size_t)n.child_ids[b]].seq_ids.front();
+  });
+  std::vector<int32_t> keys, ids;
+  for (size_t i : order) { keys.push_back(n.child_keys[i]); ids.push_back(n.child_ids[i]); }
+  n.child_keys = std::move(keys);
+  n.child_ids = std::move(ids);
+  n.key_pos.clear();
+  for (size_t i = 0; i < n.child_keys.size(); ++i) n.key_pos.emplace(n.child_keys[i], (int32_t)i);
+}
+
+void RadixPlanner::append(int seq_len, const int32_t* blocks, int n) {
+  const int seq = num_seqs();
+  insert(seq, seq_len, blocks, n);
+  seq_len_.push_back(seq_len);
+  split_per_seq_.assign(seq_len_.size(), 0);
+}
+
+void RadixPlanner::remove(int seq) {
+  if (seq < 0 || seq >= num_seqs()) throw SchedError{PAT_ERR_INDEX, "sequence index out of range"};
+  const std::vector<int> path = path_of(seq);
+  for (int node : path) {
+    auto& ids = nodes_[(size_t)node].seq_ids;
+    ids.erase(std::lower_bound(ids.begin(), ids.end(), (int32_t)seq));
+    nodes_[(size_t)node].num_seqs -= 1;
+  }
+  // rows after the removed one move up
+  for (RadixNode& n : nodes_)
+    for (int32_t& id : n.seq_ids)
+      if (id > seq) id -= 1;
+  // deepest first: nodes without sequences go, and a node left with a single child that takes all of
+  // its sequences is that child's head again (the cut that made it is undone)
+  for (size_t i = path.size(); i-- > 0;) {
+    const int node = path[i];
+    const int parent = nodes_[(size_t)node].parent;
+    if (nodes_[(size_t)node].seq_ids.empty()) {
+      // (a node without sequences has no children: each child's sequences are among its own)
+      nodes_[(size_t)parent].drop(nodes_[(size_t)node].blocks.empty() ? 0 : nodes_[(size_t)node].blocks[0]);
+      release_node(node);
+      continue;
+    }
+    RadixNode& n = nodes_[(size_t)node];
+    if (n.child_ids.size() == 1 && nodes_[(size_t)n.child_ids[0]].num_seqs == n.num_seqs) {
+      const int child = n.child_ids[0];
+      RadixNode& c = nodes_[(size_t)child];
+      n.blocks.insert(n.blocks.end(), c.blocks.begin(), c.blocks.end());
+      n.num_tokens += c.num_tokens;
+      n.child_keys = std::move(c.child_keys);
+      n.child_ids = std::move(c.child_ids);
+      n.key_pos = std::move(c.key_pos);
+      for (int grandchild : n.child_ids) nodes_[(size_t)grandchild].parent = node;
+      release_node(child);
+    }
+  }
+  // a child whose smallest sequence id was the removed one may have to move back among its siblings
+  for (int node : path)
+    if (nodes_[(size_t)node].parent != -2) sort_children(nodes_[(size_t)node].parent);
+  sort_children(0);
+  seq_len_.erase(seq_len_.begin() + seq);
+  split_per_seq_.assign(seq_len_.size(), 0);
+}
+
+void RadixPlanner::grow(int seq, int new_len, const int32_t* more_blocks, int n_more) {
+  if (seq < 0 || seq >= num_seqs()) throw SchedError{PAT_ERR_INDEX, "sequence index out of range"};
+  const int old_len = seq_len_[(size_t)seq];
+  if (new_len < old_len || n_more < 0) throw SchedError{PAT_ERR_VALUE, "a sequence can only grow"};
+  const std::vector<int> path = path_of(seq);
+  if (path.empty()) throw SchedError{PAT_ERR_VALUE, "the sequence has no blocks in the tree: build it again"};
+  const int last = path.back();
+  RadixNode& tail = nodes_[(size_t)last];
+  if (tail.seq_ids.size() == 1 && tail.child_ids.empty()) {
+    // its own leaf: more tokens, and the new blocks behind the old ones
+    tail.blocks.insert(tail.blocks.end(), more_blocks, more_blocks + n_more);
+    tail.num_tokens += new_len - old_len;
+  } else {
+    // the sequence ended on a node it shares: the new blocks become its own leaf under that node,
+    // unless they continue into one of the node's children (then only a fresh build knows the shape)
+    if (n_more == 0) {
+      if (new_len != old_len)
+        throw SchedError{PAT_ERR_VALUE, "a sequence grew inside a block it shares: build the tree again"};
+    } else {
+      if (tail.find(more_blocks[0]) >= 0)
+        throw SchedError{PAT_ERR_VALUE, "a sequence grew into blocks another one holds: build the tree again"};
+      int shared_tokens = 0;
+      for (int node : path) shared_tokens += nodes_[(size_t)node].num_tokens;
+      const int leaf = add_node(last, 1, new_len - shared_tokens, {(int32_t)seq},
+                                std::vector<int32_t>(more_blocks, more_blocks + n_more));
+      nodes_[(size_t)last].put(more_blocks[0], leaf);
+      sort_children(last);
+    }
+  }
+  seq_len_[(size_t)seq] = new_len;
+  split_per_seq_.assign(seq_len_.size(), 0);
 }
 
 // Cuts `count` sequences (ids taken from `seqs`) into boxes of at most mm sequences

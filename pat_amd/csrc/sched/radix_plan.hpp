@@ -38,6 +38,15 @@ struct RadixNode {
     auto it = key_pos.find(key);
     return it == key_pos.end() ? -1 : child_ids[it->second];
   }
+  void drop(int32_t key) {
+    auto it = key_pos.find(key);
+    if (it == key_pos.end()) return;
+    const int32_t at = it->second;
+    child_keys.erase(child_keys.begin() + at);
+    child_ids.erase(child_ids.begin() + at);
+    key_pos.clear();
+    for (size_t i = 0; i < child_keys.size(); ++i) key_pos.emplace(child_keys[i], (int32_t)i);
+  }
   void put(int32_t key, int32_t child) {
     auto it = key_pos.find(key);
     if (it == key_pos.end()) {
@@ -84,6 +93,16 @@ class RadixPlanner {
   // rows[i] = block ids of sequence i (used whole).
   void build(const int32_t* seq_lens, const int32_t* flat_blocks, const int64_t* row_offsets,
              int num_seqs);
+  // Edits of a built tree between decode steps. Each leaves the tree as build() would make it from the
+  // edited batch (same nodes, children order, sequence lists and token counts), with the split counters
+  // of a fresh tree, provided that every block two sequences share is full for both (what a paged KV
+  // cache with prefix sharing guarantees). Sequence ids are batch rows: append() adds row num_seqs(),
+  // remove() deletes a row and moves the later ones up, grow() lengthens a row in place.
+  void append(int seq_len, const int32_t* blocks, int n);
+  void remove(int seq);
+  void grow(int seq, int new_len, const int32_t* more_blocks, int n_more);
+  int num_seqs() const { return (int)seq_len_.size(); }
+
   void pack(const int32_t* mnws, int n_mnws, int hratio, int kv_heads, bool compute_model,
             const pat_sched_opts* opts);
   void naive(int hratio);
@@ -105,8 +124,14 @@ class RadixPlanner {
   void bucketize(const std::vector<Box>& boxes, const std::vector<std::vector<int32_t>>& buckets,
                  int hratio, bool force_single);
 
+  std::vector<int> path_of(int seq) const;   // nodes that hold `seq`, root's child first
+  void release_node(int node);
+  void sort_children(int node);
+
   int bs_;
   std::vector<RadixNode> nodes_;
+  std::vector<int> free_nodes_;              // slots of nodes_ given up by remove()
+  std::vector<int32_t> seq_len_;             // tokens of each sequence
   std::vector<int32_t> split_per_seq_;
   Plan plan_;
 };

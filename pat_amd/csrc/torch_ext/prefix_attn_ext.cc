@@ -609,6 +609,7 @@ struct PrefixTreeCPP {
   int block_size;
   std::vector<int32_t> batch_lens;   // the batch as build_radix_tree got it
   at::Tensor batch_table;
+  bool own_table = false;            // batch_table is a copy of ours (edits never write the caller's tensor)
   std::shared_ptr<TreeHandle> native = std::make_shared<TreeHandle>();
   std::shared_ptr<KernelInfo> info = std::make_shared<KernelInfo>();
 
@@ -639,12 +640,97 @@ struct PrefixTreeCPP {
     require(n_lens == table.size(0), "Seq lens list mismatch");
     batch_lens.assign(lens, lens + n_lens);
     batch_table = table;
+    own_table = false;
     int rc;
     {
       py::gil_scoped_release release;   // the tree is built without the GIL (csrc/bindings.cpp:124)
       rc = pat_tree_build(native->h, lens, table.data_ptr<int32_t>(), (int32_t)table.size(0), (int32_t)table.size(1));
     }
     check(rc);
+  }
+
+  // ---- edits between decode steps (include/pat_amd.h: pat_tree_append / _remove / _grow) -----------
+  // The batch copy (lengths and block rows: what the whole-sequence tables are made from) follows.
+  void set_row(int64_t row, const std::vector<int32_t>& blocks, int64_t first) {
+    const int64_t need = first + (int64_t)blocks.size();
+    if (!batch_table.defined() || batch_table.size(1) < need) {
+      const int64_t rows = batch_table.defined() ? batch_table.size(0) : 0;
+      at::Tensor wider = at::zeros({rows, need + 8}, at::TensorOptions().dtype(at::kInt));
+      if (rows > 0 && batch_table.size(1) > 0)
+        wider.slice(1, 0, batch_table.size(1)).copy_(batch_table);
+      batch_table = wider;
+      own_table = true;
+    }
+    if (!own_table) { batch_table = batch_table.clone(); own_table = true; }
+    int32_t* dst = batch_table.data_ptr<int32_t>() + row * batch_table.size(1) + first;
+    for (size_t i = 0; i < blocks.size(); ++i) dst[i] = blocks[i];
+  }
+
+  int64_t append_sequence(int seq_len, const std::vector<int32_t>& blocks) {
+    check(pat_tree_append(native->h, seq_len, blocks.data(), (int32_t)blocks.size()));
+    const int64_t row = (int64_t)batch_lens.size();
+    const int64_t width = std::max<int64_t>(batch_table.defined() ? batch_table.size(1) : 0, (int64_t)blocks.size());
+    at::Tensor taller = at::zeros({row + 1, width}, at::TensorOptions().dtype(at::kInt));
+    if (row > 0 && batch_table.defined() && batch_table.size(1) > 0)
+      taller.slice(0, 0, row).slice(1, 0, batch_table.size(1)).copy_(batch_table);
+    batch_table = taller;
+    own_table = true;
+    batch_lens.push_back(seq_len);
+    set_row(row, blocks, 0);
+    return row;
+  }
+
+  void remove_sequence(int seq) {
+    check(pat_tree_remove(native->h, seq));
+    const int64_t rows = (int64_t)batch_lens.size();
+    batch_lens.erase(batch_lens.begin() + seq);
+    if (batch_table.defined() && batch_table.size(0) == rows)
+      batch_table = at::cat({batch_table.slice(0, 0, seq), batch_table.slice(0, seq + 1, rows)}, 0).contiguous();
+    own_table = true;
+  }
+
+  void grow_sequence(int seq, int new_len, const std::vector<int32_t>& more_blocks) {
+    require(seq >= 0 && (size_t)seq < batch_lens.size(), "sequence index out of range");
+    check(pat_tree_grow(native->h, seq, new_len, more_blocks.data(), (int32_t)more_blocks.size()));
+    const int64_t had = ((int64_t)batch_lens[(size_t)seq] + block_size - 1) / block_size;
+    batch_lens[(size_t)seq] = new_len;
+    if (!more_blocks.empty()) set_row(seq, more_blocks, had);
+  }
+
+  // One decode step later: same rows, each with its new length and the block row of the step's
+  // metadata (rows grow by appending blocks). Grows every row in place; when a row cannot be grown
+  // (see pat_tree_grow) the tree is built afresh from the arguments. Returns true when no rebuild
+  // was needed. Either way the tree is that of build_radix_tree(seq_lens, block_table).
+  bool advance(const std::vector<int32_t>& seq_lens, const at::Tensor& table_in) {
+    require(table_in.dim() == 2 && table_in.device().is_cpu() && table_in.scalar_type() == at::kInt,
+            "block_table must be a 2-D CPU Int32 Tensor");
+    require((int64_t)seq_lens.size() == table_in.size(0), "Seq lens list mismatch");
+    const at::Tensor table = table_in.contiguous();
+    bool grown = seq_lens.size() == batch_lens.size();
+    if (grown) {
+      py::gil_scoped_release release;
+      const int32_t* t = table.data_ptr<int32_t>();
+      const int64_t w = table.size(1);
+      for (size_t i = 0; i < seq_lens.size() && grown; ++i) {
+        if (seq_lens[i] == batch_lens[i]) continue;
+        const int64_t had = ((int64_t)batch_lens[i] + block_size - 1) / block_size;
+        const int64_t need = ((int64_t)seq_lens[i] + block_size - 1) / block_size;
+        if (seq_lens[i] < batch_lens[i] || need > w) { grown = false; break; }
+        grown = pat_tree_grow(native->h, (int32_t)i, seq_lens[i], t + (int64_t)i * w + had, (int32_t)(need - had)) == PAT_OK;
+      }
+    }
+    if (!grown) {
+      int rc;
+      {
+        py::gil_scoped_release release;
+        rc = pat_tree_build(native->h, seq_lens.data(), table.data_ptr<int32_t>(), (int32_t)table.size(0), (int32_t)table.size(1));
+      }
+      check(rc);
+    }
+    batch_lens = seq_lens;
+    batch_table = table;
+    own_table = false;
+    return grown;
   }
 
   void pack_schedule(const py::object& mnws_obj, int hratio, int kv_head, bool use_compute_model) {
@@ -974,6 +1060,18 @@ PYBIND11_MODULE(_prefix_attn, m) {
       .def(py::init<int>(), py::arg("block_size"))
       .def_readonly("block_size", &PrefixTreeCPP::block_size)
       .def("build_radix_tree", &PrefixTreeCPP::build_radix_tree, py::arg("seq_lens"), py::arg("block_table"))
+      .def("append_sequence", &PrefixTreeCPP::append_sequence, py::arg("seq_len"), py::arg("blocks"),
+           "A request joins the batch behind the last row; returns its row. The tree is then what "
+           "build_radix_tree gives for the edited batch.")
+      .def("remove_sequence", &PrefixTreeCPP::remove_sequence, py::arg("seq"),
+           "Row `seq` leaves the batch; the rows behind it move up by one.")
+      .def("grow_sequence", &PrefixTreeCPP::grow_sequence, py::arg("seq"), py::arg("new_len"),
+           py::arg("more_blocks") = std::vector<int32_t>(),
+           "Row `seq` now has new_len tokens and `more_blocks` behind its old blocks. Raises ValueError (tree "
+           "unchanged) when only a fresh build can know the new shape.")
+      .def("advance", &PrefixTreeCPP::advance, py::arg("seq_lens"), py::arg("block_table"),
+           "One decode step later: the same rows with their new lengths and block rows. Grows the tree in place "
+           "(False: it had to be built afresh); the result equals build_radix_tree(seq_lens, block_table).")
       .def("pack_schedule", &PrefixTreeCPP::pack_schedule, py::arg("MNWs") = py::none(), py::arg("HRatio") = 1,
            py::arg("kvHead") = 8, py::arg("use_compute_model") = false)
       .def_property_readonly("kernel_info", [](const PrefixTreeCPP& t) { return t.info; });

@@ -89,6 +89,20 @@ class _NativeTree:
         _lib.check(self._lib.pat_tree_build(self._h, _ptr(seq_lens), _ptr(table),
                                             int(table.shape[0]), int(table.shape[1])))
 
+    def append(self, seq_len: int, blocks: Sequence[int]) -> None:
+        b = _as_i32(list(blocks))
+        _lib.check(self._lib.pat_tree_append(self._h, int(seq_len), _ptr(b), int(b.size)))
+
+    def remove(self, seq: int) -> None:
+        _lib.check(self._lib.pat_tree_remove(self._h, int(seq)))
+
+    def grow(self, seq: int, new_len: int, more_blocks: Sequence[int]) -> None:
+        b = _as_i32(list(more_blocks))
+        _lib.check(self._lib.pat_tree_grow(self._h, int(seq), int(new_len), _ptr(b), int(b.size)))
+
+    def num_seqs(self) -> int:
+        return self._lib.pat_tree_num_seqs(self._h)
+
     def pack(self, MNWs, HRatio: int, kvHead: int, use_compute_model: bool, opts=None) -> None:
         if MNWs is None:
             arr, n = None, 0
@@ -137,6 +151,28 @@ class PrefixTree:
         """Inserts row i of `block_table` (used whole) with length seq_lens[i], in order."""
         self._native.build_rows(seq_lens, block_table)
         self.split_per_seq = [0] * len(block_table)
+
+    # -- edits between decode steps (no counterpart in the reference, which builds a new tree per
+    #    step: plugin/vllm/attention/backends/prefix_attn.py:330-338). After any of them the tree and
+    #    the plans packed from it are those of a fresh build_radix_tree on the edited batch, provided
+    #    every block two requests share is full for both. --------------------------------------------
+    def append_sequence(self, seq_len: int, blocks: List[int]) -> int:
+        """A request joins the batch behind the last row; returns its row."""
+        self._native.append(seq_len, blocks)
+        self.split_per_seq = [0] * self._native.num_seqs()
+        return len(self.split_per_seq) - 1
+
+    def remove_sequence(self, seq: int) -> None:
+        """Row `seq` leaves the batch; the rows behind it move up by one."""
+        self._native.remove(seq)
+        self.split_per_seq = [0] * self._native.num_seqs()
+
+    def grow_sequence(self, seq: int, new_len: int, more_blocks: Sequence[int] = ()) -> None:
+        """Row `seq` now has new_len tokens and the blocks `more_blocks` behind its old ones. Raises
+        ValueError (tree unchanged) when only a fresh build can know the new shape: the row grew inside a
+        block it shares, or into blocks another row holds."""
+        self._native.grow(seq, new_len, more_blocks)
+        self.split_per_seq = [0] * self._native.num_seqs()
 
     # -- scheduling -------------------------------------------------------------
     def pack_schedule(self, MNWs: Optional[List[List[int]]] = None, HRatio: int = 1, kvHead: int = 8,

@@ -17,6 +17,10 @@ AttentionMetadata) can drive:
   (and, at a page boundary, the next block id) in place on the device; the plan is rebuilt only
   when that is not possible (a tail shared by several requests, a block row that is full).
 
+* `DecodePlan.from_previous(prev, meta, left, joined)` makes the next step's plan by editing the
+  previous step's tree (requests that left, requests that joined, every row one step longer)
+  instead of building a new tree; the result is the plan a fresh build gives.
+
 `meta` only needs the attributes read here (`num_prefills`, `num_decode_tokens`, `seq_lens`,
 `block_tables`, `block_tables_cpu`, `block_size`, `nheads`, `nheads_kv`,
 `max_decode_query_len`); vLLM's own metadata class has them after the reference's overlay.
@@ -63,6 +67,35 @@ class DecodePlan:
         device = tables.device if tables is not None else torch.device("cuda")
         tree = AsyncTree(block_size=meta.block_size, seq_lens=seq_lens, table=table_cpu, MNWs=None,
                          HRatio=meta.nheads // meta.nheads_kv, kvHead=meta.nheads_kv, device=device)
+        return cls(num_decode_tokens=meta.num_decode_tokens, seq_lens=seq_lens, block_tables=tables, tree=tree,
+                   max_decode_query_len=getattr(meta, "max_decode_query_len", 1), block_size=meta.block_size,
+                   nheads=meta.nheads, nheads_kv=meta.nheads_kv)
+
+    @classmethod
+    def from_previous(cls, prev: "DecodePlan", meta: Any, left: List[int] = (), joined: int = 0) -> "DecodePlan":
+        """The next step's plan made by editing the previous step's tree instead of building a new one
+        (the reference builds one per step, `decode_metadata` :313-338). `left`: rows of the previous
+        decode batch that are gone; the requests that stay keep their order and the `joined` new ones
+        stand behind them in `meta` (vLLM appends to its running queue). Every remaining row's new
+        length and block row come from `meta`. The tree and the plan are those a fresh build gives for
+        this batch (`pat_tree_remove` / `pat_tree_append` / `pat_tree_grow`); rows that cannot be
+        grown in place make the tree fall back to a fresh build by itself."""
+        first = meta.num_prefills
+        seq_lens = list(meta.seq_lens[first:])
+        tables = None if meta.block_tables is None else meta.block_tables[first:]
+        table_cpu = meta.block_tables_cpu[first:] if meta.block_tables_cpu.shape[0] != len(seq_lens) \
+            else meta.block_tables_cpu
+        tree = prev._ready_tree()
+        for row in sorted(left, reverse=True):
+            tree.remove_sequence(int(row))
+        stay = len(seq_lens) - joined
+        bs = meta.block_size
+        for row in range(stay, len(seq_lens)):
+            tree.append_sequence(int(seq_lens[row]), table_cpu[row, :-(-int(seq_lens[row]) // bs)].tolist())
+        tree.advance(seq_lens, table_cpu)
+        tree.pack_schedule(MNWs=None, HRatio=meta.nheads // meta.nheads_kv, kvHead=meta.nheads_kv)
+        device = tables.device if tables is not None else prev._ready_tree().kernel_info.num_split_per_seq.device
+        tree.kernel_info.to_gpu(device)
         return cls(num_decode_tokens=meta.num_decode_tokens, seq_lens=seq_lens, block_tables=tables, tree=tree,
                    max_decode_query_len=getattr(meta, "max_decode_query_len", 1), block_size=meta.block_size,
                    nheads=meta.nheads, nheads_kv=meta.nheads_kv)

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"libpat_amd.so does not export {name}"
     assert sorted(_lib.SYMBOLS) == names       # the ctypes table covers the header, no more, no less
-    assert lib.pat_abi_version() == 3
+    assert lib.pat_abi_version() == 4
 
 
 def _args(**over):

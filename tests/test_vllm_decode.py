@@ -241,8 +241,9 @@ def test_fifty_replanned_decode_steps_with_requests_leaving_and_joining():
     output = torch.empty_like(query)
     width = w.padded_table().shape[1] + 8
 
-    def serve(tuning_on):
+    def serve(tuning_on, incremental=False):
         rows, lens = [list(r) for r in w.rows], list(w.seq_lens)
+        plan = None
         spare = iter(range(w.num_blocks, w.num_blocks + spare_blocks))
         ext.set_autotune(tuning_on)
         ext.clear_autotune_cache()
@@ -254,16 +255,26 @@ def test_fifty_replanned_decode_steps_with_requests_leaving_and_joining():
                     if lens[i] % page == 0:
                         rows[i].append(next(spare))
                     lens[i] += 1
-                if step % 5 == 0:                              # one leaves, one joins on its row
+                left, joined = [], 0
+                if step % 5 == 0:                              # one leaves, one joins
                     i = (7 * step) % w.batch
                     fresh = 64 + (37 * step) % 448
-                    rows[i] = rows[i][:prefix] + [next(spare) for _ in range(-(-fresh // page))]
-                    lens[i] = prefix * page + fresh
+                    blocks = rows[i][:prefix] + [next(spare) for _ in range(-(-fresh // page))]
+                    if incremental:                            # (behind the others, as vLLM queues it)
+                        del rows[i], lens[i]
+                        rows.append(blocks)
+                        lens.append(prefix * page + fresh)
+                        left, joined = [i], 1
+                    else:                                      # (on the row that became free)
+                        rows[i], lens[i] = blocks, prefix * page + fresh
                 table = _table(rows, width)
                 meta = SimpleNamespace(num_prefills=0, num_decode_tokens=w.batch, seq_lens=list(lens),
                                        block_tables=table.to(dev), block_tables_cpu=table, block_size=page,
                                        nheads=w.heads, nheads_kv=w.kv_heads, max_decode_query_len=1)
-                plan = DecodePlan.from_metadata(meta)
+                if incremental and plan is not None:
+                    plan = DecodePlan.from_previous(plan, meta, left, joined)
+                else:
+                    plan = DecodePlan.from_metadata(meta)
                 decode_attention(query, kv_cache, plan, 1.0 / math.sqrt(w.head_dim), output)
                 if step in (1, 5, 26, 50):
                     torch.cuda.synchronize()
@@ -278,7 +289,50 @@ def test_fifty_replanned_decode_steps_with_requests_leaving_and_joining():
 
     runs, worst = serve(False)
     print(f"[parity] default settings: {runs} tuning runs, max|out - ref| = {worst:.3e}", flush=True)
+    runs_inc, worst_inc = serve(False, incremental=True)
+    print(f"[parity] plans made by editing the previous step's tree: max|out - ref| = {worst_inc:.3e}", flush=True)
+    assert runs_inc == 0
     assert runs == 0
     runs, worst = serve(True)
     print(f"[parity] tuning switched on: {runs} tuning runs over {steps} plans, max|out - ref| = {worst:.3e}", flush=True)
     assert runs <= 4
+
+
+def test_next_step_plan_from_the_previous_tree_equals_a_fresh_one():
+    """DecodePlan.from_previous edits the previous step's tree (rows gone, rows joined, every row a
+    token longer): plan tables equal those of a plan built from the step's metadata alone."""
+    w = workloads.make("c2", seed=8)
+    page = w.page_size
+    rows, lens, nxt = [list(r) for r in w.rows], list(w.seq_lens), w.num_blocks
+
+    def meta_of():
+        t = _table(rows, 180)
+        return SimpleNamespace(num_prefills=0, num_decode_tokens=len(rows), seq_lens=list(lens), block_tables=t,
+                               block_tables_cpu=t, block_size=page, nheads=w.heads, nheads_kv=w.kv_heads,
+                               max_decode_query_len=1)
+
+    plan = DecodePlan.from_metadata(meta_of())
+    for step in range(1, 21):
+        left, joined = [], 0
+        for i in range(len(rows)):
+            if lens[i] % page == 0:
+                rows[i].append(nxt)
+                nxt += 1
+            lens[i] += 1
+        if step % 5 == 0:
+            i = (7 * step) % len(rows)
+            left = [i]
+            del rows[i], lens[i]
+            fresh = 64 + (37 * step) % 448
+            rows.append(rows[0][:2048 // page] + list(range(nxt, nxt + -(-fresh // page))))
+            nxt += -(-fresh // page)
+            lens.append(2048 + fresh)
+            joined = 1
+        meta = meta_of()
+        plan = DecodePlan.from_previous(plan, meta, left, joined)
+        fresh_plan = DecodePlan.from_metadata(meta)
+        got, want = plan.tree.kernel_info, fresh_plan.tree.tree.kernel_info
+        assert got.num_split_per_seq.tolist() == want.num_split_per_seq.tolist()
+        for name in ("q_tables", "num_seqs_per_CTAs", "CTA_ranks", "kv_in_CTAs", "block_tables"):
+            for x, y in zip(getattr(got, name), getattr(want, name)):
+                assert torch.equal(x, y), (step, name)
