@@ -17,7 +17,8 @@ latency per call: W warm-up steps, then the K timed steps between two synchronis
 duration = mean split-kernel time from HIP events on the launch stream. `autotune` reports what
 the optional measured choice of the geometry (pat_fwd_autotune, off by default in the product)
 would give and what measuring costs; `records_build_us` the kernel that turns the plan tables into
-launch records once per plan; `plan_build_ms_host` the host planner in steady state.
+launch records once per plan; `plan_build_ms_host` the host planner in steady state (tree + pack +
+flat tables); `tree_next_step_ms_host` the next decode step's tree edited in place against built anew.
 `cpu_baseline` times this repository's CPU restatement of the reference's PyTorch attention
 on the host cores. `api_us_per_call` is the same loop through the drop-in call
 `prefix_attn_with_kvcache(q, k, v, tree, scale, out)` of the compiled extension (workspace from
@@ -112,12 +113,38 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
     q, ks, vs = w.tensors(dev, copies=copies)
     scale = 1.0 / math.sqrt(w.head_dim)
 
+    batch_table = w.padded_table()     # (what a serving loop has at hand: the step's CPU block table)
+
     def plan():
         t0 = time.perf_counter()
         tree = PrefixTreeCPP(w.page_size)
-        tree.build_radix_tree(w.seq_lens, w.padded_table())
+        tree.build_radix_tree(w.seq_lens, batch_table)
         tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
         return tree, (time.perf_counter() - t0) * 1e3
+
+    def plan_next_step():
+        # the tree of the next decode step (every request a token longer) made by editing this step's
+        # tree (PrefixTreeCPP.advance) against building it anew; median of 5, milliseconds
+        tree = PrefixTreeCPP(w.page_size)
+        table = torch.cat([batch_table, torch.zeros(w.batch, 2, dtype=torch.int32)], dim=1)
+        lens = list(w.seq_lens)
+        tree.build_radix_tree(lens, table)
+        spare, edit, build = w.num_blocks, [], []
+        for _ in range(5):
+            for i in range(w.batch):
+                if lens[i] % w.page_size == 0:
+                    table[i, lens[i] // w.page_size] = spare
+                    spare += 1
+                lens[i] += 1
+            t0 = time.perf_counter()
+            in_place = tree.advance(lens, table)
+            edit.append((time.perf_counter() - t0) * 1e3)
+            assert in_place
+            fresh = PrefixTreeCPP(w.page_size)
+            t0 = time.perf_counter()
+            fresh.build_radix_tree(lens, table)
+            build.append((time.perf_counter() - t0) * 1e3)
+        return sorted(edit)[2], sorted(build)[2]
 
     _, plan_first_ms = plan()          # (the first call also pays for the pinned buffer pool)
     plan_runs = sorted(plan()[1] for _ in range(5))
@@ -275,6 +302,7 @@ def measure(a, workload: str, steps: int, warmup: int, headline: bool) -> dict:
                      "chunks_per_rank": geo.chunks_per_rank, "workgroups": geo.num_workgroups},
         "plan_build_ms_host": round(plan_ms, 3),
         "plan_build_first_call_ms": round(plan_first_ms, 3),
+        "tree_next_step_ms_host": dict(zip(("edited_in_place", "built_anew"), (round(x, 4) for x in plan_next_step()))),
         "records_build_us": round(records_build_us, 2),
         "autotune": None,
         "roofline": {"bound": "hbm", "kernel": "pat_split_kernel", "achieved": round(achieved, 2),
