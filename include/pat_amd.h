@@ -278,6 +278,10 @@ typedef struct pat_fwd_tuning {
   int32_t equalize_chunks;           /* even chunks per box: -1 automatic, 0 never, 1 always        */
   int32_t direct_out;                /* single-slot launches write `out` from the split kernel:     */
                                      /* -1 / 1 when possible, 0 never                               */
+  int32_t tall_rows;                 /* rows per wave on boxes of 17..64 rows: 32 (32x32x16 MFMA    */
+                                     /* tiles, 2 workgroups per CU at head_dim 128), 16 (16x16x32,  */
+                                     /* 3 per CU), 0: chosen per launch from its sizes              */
+  int32_t reserved;                  /* 0                                                           */
 } pat_fwd_tuning;
 int pat_fwd_set_tuning(const pat_fwd_tuning* tuning);
 int pat_fwd_get_tuning(pat_fwd_tuning* out);
@@ -430,6 +434,8 @@ typedef struct pat_fwd_geometry {
   int32_t chunks_per_rank;   /* partial slots reserved per box                     */
   int32_t num_slots;         /* max_split_per_seq * chunks_per_rank                */
   int64_t num_workgroups;    /* split-kernel workgroups                            */
+  int32_t tall_rows;         /* form of the tall path: 32 or 16 rows per wave      */
+  int32_t reserved;
 } pat_fwd_geometry;
 int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out);
 

@@ -100,11 +100,11 @@ class FwdTuning(C.Structure):
     _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
                 ("head_per_wave_tokens", C.c_int32), ("head_per_wave_long_tokens", C.c_int32),
                 ("head_per_wave_long_wgs", C.c_int64), ("equalize_chunks", C.c_int32),
-                ("direct_out", C.c_int32)]
+                ("direct_out", C.c_int32), ("tall_rows", C.c_int32), ("reserved", C.c_int32)]
 
     @classmethod
     def automatic(cls) -> "FwdTuning":
-        return cls(0, 0, -1, 0, -1, -1, -1)
+        return cls(0, 0, -1, 0, -1, -1, -1, 0, 0)
 
 
 class FwdArgs(C.Structure):
@@ -127,7 +127,7 @@ class FwdArgs(C.Structure):
 class FwdGeometry(C.Structure):
     _fields_ = [("chunk_tokens", C.c_int32), ("tall_chunk_tokens", C.c_int32),
                 ("chunks_per_rank", C.c_int32), ("num_slots", C.c_int32),
-                ("num_workgroups", C.c_int64)]
+                ("num_workgroups", C.c_int64), ("tall_rows", C.c_int32), ("reserved", C.c_int32)]
 
 
 # Every symbol include/pat_amd.h declares: name -> (restype, argtypes)

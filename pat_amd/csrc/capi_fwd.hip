@@ -29,8 +29,9 @@ constexpr int kMaxChunk = 2048;
 constexpr int kTallChunk = 256;
 constexpr int kSmallLaunchTokens = 512;      // boxes up to this length stay whole in launches of less than a workgroup per CU
 constexpr int kLongHeadPerWaveChunk = 1024;   // tokens a wave walks alone (long boxes, a kv head per wave)
-// workgroups of the split kernel a CU holds at once: head_dim 128 -> 2 (registers and LDS of the 32-row tiles), 64 -> 3
-inline int resident_wgs_per_cu(int head_dim) { return head_dim == 128 ? 2 : 3; }
+// workgroups of the split kernel a CU holds at once: 3, or 2 at head_dim 128 with 32-row tiles on tall boxes
+// (their registers and LDS)
+inline int resident_wgs_per_cu(int head_dim, int tall_rows) { return (head_dim == 128 && tall_rows == 32) ? 2 : 3; }
 
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t gcd64(int64_t a, int64_t b) { while (b) { int64_t t = a % b; a = b; b = t; } return a; }
@@ -43,12 +44,14 @@ inline int row_tiles(int m_label) { return m_label <= 16 ? 1 : (m_label <= 32 ? 
 
 // Overrides of the launch geometry (pat_fwd_set_tuning). The defaults come from the environment
 // variables PAT_CHUNK_TOKENS, PAT_TALL_CHUNK_TOKENS, PAT_HEAD_PER_WAVE_TOKENS,
-// PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS, PAT_EQUALIZE_CHUNKS and
-// PAT_DIRECT_OUT, read once per process: no launch reads the environment.
+// PAT_HEAD_PER_WAVE_LONG_WGS, PAT_HEAD_PER_WAVE_LONG_TOKENS, PAT_EQUALIZE_CHUNKS, PAT_DIRECT_OUT and
+// PAT_TALL_ROWS, read once per process: no launch reads the environment.
 pat_fwd_tuning env_tuning() {
   pat_fwd_tuning t;
   t.chunk_tokens = 0; t.tall_chunk_tokens = 0; t.head_per_wave_tokens = -1;
   t.head_per_wave_long_wgs = -1; t.head_per_wave_long_tokens = 0; t.equalize_chunks = -1; t.direct_out = -1;
+  t.tall_rows = 0; t.reserved = 0;
+  if (const char* e = std::getenv("PAT_TALL_ROWS")) t.tall_rows = std::atoi(e);
   if (const char* e = std::getenv("PAT_CHUNK_TOKENS")) t.chunk_tokens = std::atoi(e);
   if (const char* e = std::getenv("PAT_TALL_CHUNK_TOKENS")) t.tall_chunk_tokens = std::atoi(e);
   if (const char* e = std::getenv("PAT_HEAD_PER_WAVE_TOKENS")) t.head_per_wave_tokens = std::atoi(e);
@@ -82,6 +85,7 @@ struct Geometry {
   int bucket_chunks[kMaxBuckets] = {0};
   int bucket_heads_per_wg[kMaxBuckets] = {0};   // 1, or kWaves: one kv head per wave
   int64_t total_wgs = 0;
+  int tall_rows = 32;        // rows per wave on boxes of 17..64 rows: 32 or 16 (the split kernel's instance)
   bool direct = false;       // one slot per row: the split kernel writes `out`, no workspace, no merge kernel
   // launch records (one per workgroup): entries per record and bytes between records
   int record_max_seqs = 0, record_max_pages = 0, record_stride = 0;
@@ -180,7 +184,23 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
     const int64_t w = (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
     if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w;
   }
-  const int64_t resident = (int64_t)resident_wgs_per_cu(a->head_dim) * kNumCUs;
+  // Which form of the tall path (boxes of 17..64 rows): 32-row tiles walk a tall box faster and cost a
+  // resident workgroup per CU at head_dim 128; they pay where the launch waits for its tall boxes.
+  // Estimated from sizes: a tall workgroup takes ~1.25 us per 64 tokens, the <= 16-row boxes stream at
+  // ~5.8 TB/s, ragged buckets (no PAT_BUCKET_EVEN hint) hold ~0.6 of their widest box on average.
+  int tall_rows = tune.tall_rows == 16 || tune.tall_rows == 32 ? tune.tall_rows : 0;
+  if (tall_rows == 0) {
+    double tall_us = 0., short_us = 0.;
+    for (int i = 0; i < a->num_buckets; ++i) {
+      const pat_fwd_bucket& b = a->buckets[i];
+      const double token_heads = (double)b.max_blocks * page * b.num_boxes * a->kv_heads;
+      if (row_tiles(b.mnw[0]) > 1) tall_us += token_heads / 64. * 1.25 / kNumCUs;
+      else short_us += token_heads * ((b.flags & PAT_BUCKET_EVEN) ? 1.0 : 0.6) * a->head_dim * 4. / 5.8e6;
+    }
+    tall_rows = tall_us > 0. && tall_us >= short_us ? 32 : 16;
+  }
+  g->tall_rows = tall_rows;
+  const int64_t resident = (int64_t)resident_wgs_per_cu(a->head_dim, tall_rows) * kNumCUs;
   int64_t chunk = tune.chunk_tokens, tall = tune.tall_chunk_tokens;
   const bool env_tall = tall > 0, env_chunk = chunk > 0;
   if (chunk <= 0) {
@@ -202,7 +222,9 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
         tall_box_heads += (int64_t)a->buckets[i].num_boxes * a->kv_heads;
         widest_tall = std::max<int64_t>(widest_tall, (int64_t)a->buckets[i].max_blocks * page);
       }
-    const int64_t pieces = tall_box_heads > 0 ? std::max<int64_t>(1, ceil_div64(3 * kNumCUs / 8, tall_box_heads)) : 1;
+    // (the 16-row form's steps are slower: it wants a tall workgroup per two CUs)
+    const int64_t want_tall_wgs = tall_rows == 32 ? 3 * kNumCUs / 8 : kNumCUs / 2;
+    const int64_t pieces = tall_box_heads > 0 ? std::max<int64_t>(1, ceil_div64(want_tall_wgs, tall_box_heads)) : 1;
     tall = ceil_div64(ceil_div64(widest_tall, pieces), 128) * 128;
     tall = std::max<int64_t>(kTallChunk, std::min<int64_t>(kMaxChunk, tall));
   }
@@ -387,7 +409,7 @@ size_t workspace_need(const pat_fwd_args* a, const Geometry& g) {
 uint64_t records_tag(const pat_fwd_args* a, const Geometry& g) {
   uint64_t h = 0x9e3779b97f4a7c15ull;
   auto mix = [&](uint64_t v) { h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2); };
-  mix((uint64_t)g.total_wgs); mix((uint64_t)g.record_stride); mix((uint64_t)g.record_max_seqs); mix((uint64_t)g.record_max_pages);
+  mix((uint64_t)g.tall_rows); mix((uint64_t)g.total_wgs); mix((uint64_t)g.record_stride); mix((uint64_t)g.record_max_seqs); mix((uint64_t)g.record_max_pages);
   mix((uint64_t)g.num_slots); mix((uint64_t)g.chunks_per_rank); mix(g.direct ? 1 : 0);
   mix((uint64_t)a->batch); mix((uint64_t)a->heads); mix((uint64_t)a->kv_heads); mix((uint64_t)a->page_size);
   mix((uint64_t)a->num_pages); mix((uint64_t)a->max_split_per_seq);
@@ -422,6 +444,8 @@ int pat_fwd_geometry_of(const pat_fwd_args* args, pat_fwd_geometry* out) {
   out->chunks_per_rank = g.chunks_per_rank;
   out->num_slots = g.num_slots;
   out->num_workgroups = g.total_wgs;
+  out->tall_rows = g.tall_rows;
+  out->reserved = 0;
   return PAT_OK;
 }
 
@@ -582,6 +606,7 @@ int launch_core(const pat_fwd_args* args, const Geometry& g, void* workspace, vo
   sp.q = args->q; sp.k = args->k; sp.v = args->v;
   sp.o_part = o_part; sp.lse_part = lse_part;
   sp.direct = g.direct ? 1 : 0;
+  sp.tall_rows = g.tall_rows;
   if (g.direct) {
     sp.out = args->out; sp.lse_out = args->lse_out;
     sp.o_stride_b = args->o_stride[0]; sp.o_stride_h = args->o_stride[2];
@@ -827,6 +852,7 @@ pat_fwd_tuning automatic_tuning() {
   pat_fwd_tuning t;
   t.chunk_tokens = 0; t.tall_chunk_tokens = 0; t.head_per_wave_tokens = -1; t.head_per_wave_long_tokens = 0;
   t.head_per_wave_long_wgs = -1; t.equalize_chunks = -1; t.direct_out = -1;
+  t.tall_rows = 0; t.reserved = 0;
   return t;
 }
 // Candidates beside the automatic geometry: a kv head per wave on <= 16-row boxes in chunks of 256

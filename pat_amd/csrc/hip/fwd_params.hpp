@@ -54,6 +54,7 @@ struct SplitParams {
   float* lse_out;    // optional [batch, heads] fp32
   int64_t o_stride_b, o_stride_h;              // elements
   int32_t direct;    // 1: such a launch
+  int32_t tall_rows; // rows per wave on boxes of 17..64 rows: 32 (32x32x16 tiles) or 16 (host side: picks the kernel instance)
 };
 
 // One tile bucket as the record kernel sees it.

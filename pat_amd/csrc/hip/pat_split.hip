@@ -84,23 +84,31 @@ __device__ __forceinline__ float neg_inf() { return -__builtin_inff(); }
 #define PAT_DEPTH 1
 #endif
 
-// Resident workgroups per CU the register budget is sized for. head_dim 128: the tall path holds
-// 32 rows x 128 columns of O^T per wave (64 registers) beside Q (32) and two super-steps of
-// prefetch (64): 2 workgroups; head_dim 64 fits 3.
-__host__ __device__ constexpr int split_occupancy(int head_dim) { return head_dim == 128 ? 2 : 3; }
+// Two forms of the tall path (boxes of 17..64 rows), one kernel instance each:
+//  TALLK 32: 32-row tiles on 32x32x16 MFMAs, 64-token super-steps; the faster walk of a tall box
+//            (a lone workgroup: 1.1-1.3 us per 64 tokens), at the price of 64 accumulator registers
+//            and 75 KB of LDS: 2 workgroups per CU at head_dim 128;
+//  TALLK 16: a 16-row tile per wave on 16x16x32 MFMAs, 32-token steps, three steps ahead in registers
+//            (1.7 us per 64 tokens), in the register and LDS budget of the <= 16-row path: 3 per CU.
+// The host picks per launch: 32 where the tall boxes are what the launch waits for, 16 where the
+// <= 16-row boxes are and the third resident workgroup per CU is worth more (pat_fwd_tuning.tall_rows).
+__host__ __device__ constexpr int split_occupancy(int head_dim, int tallk) {
+  return (head_dim == 128 && tallk == 32) ? 2 : 3;
+}
 
 // LDS bytes of one workgroup (dynamic: more than the 64 KB a static allocation may have).
-__host__ __device__ constexpr int split_smem_bytes(int D) {
+__host__ __device__ constexpr int split_smem_bytes(int D, int tallk) {
   const int wave_private = kWaves * kStepTokens * (D * 2 + 32);     // 4 private V tiles
   const int combine = kWaves * 16 * (D + 4) * 4;                     // short boxes: the waves' states
-  const int tall = 2 * (2 * kStepTokens) * ((D * 2 + 16) + (D * 2 + 64));   // two stages of 64 K rows + 64 V rows
+  const int tall = tallk == 32 ? 2 * (2 * kStepTokens) * ((D * 2 + 16) + (D * 2 + 64))   // two stages of 64 K rows + 64 V rows
+                               : 2 * kStepTokens * ((D * 2 + 16) + (D * 2 + 32));        // two stages of 32 K rows + 32 V rows
   int m = wave_private > combine ? wave_private : combine;
   return m > tall ? m : tall;
 }
 
 // DIRECT instances serve launches in which every row has one partial slot: they store `out`.
-template <typename T, int D, bool DIRECT>
-__global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel(const char* __restrict__ records, const int record_stride,
+template <typename T, int D, bool DIRECT, int TALLK>
+__global__ void __launch_bounds__(kThreads, split_occupancy(D, TALLK)) pat_split_kernel(const char* __restrict__ records, const int record_stride,
                                                                              const int record_max_seqs, const SplitParams p) {
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -166,7 +174,7 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
   const int gshift = 31 - __builtin_clz(G);
   const int page = p.page_size;
   // this lane's row: sequence id and partial-result slot (-1: no such row)
-  const int my_row = tall ? rt * 32 + n32 : n;
+  const int my_row = tall ? (TALLK == 32 ? rt * 32 + n32 : wave * 16 + n) : n;
   const int my_j = my_row >> gshift;
   const bool j_ok = (my_row < R) && my_j < record_max_seqs;
   const int* __restrict__ rows_tab = (const int*)(rec + sizeof(RecordHead));
@@ -179,13 +187,13 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
   const int pg0 = (lane < npages) ? pages_tab[lane] : 0;
   const int pg1 = (64 + lane < npages) ? pages_tab[64 + lane] : 0;
 
-  const bool has_rows = !tall || rt * 32 < R;   // false: a wave that only helps loading shared tiles
+  const bool has_rows = !tall || (TALLK == 32 ? rt * 32 : wave * 16) < R;   // false: a wave that only helps loading shared tiles
   const bool row_ok = my_seq >= 0 && my_sl >= 0;
   const int my_hq = head * G + (my_row & (G - 1));
   // partial slot of (my row, this piece); -1: the row is not to be written
   const int my_slot0 = row_ok ? (my_seq * p.heads + my_hq) * p.num_slots + my_sl : -1;
   // the one lane per row that writes what exists once per row (LSE, empty-slot marks)
-  const bool row_lead = tall ? (ph == 0 && h2 == 0) : ((head_per_wave || wave == 0) && g == 0);
+  const bool row_lead = tall ? (TALLK == 32 ? (ph == 0 && h2 == 0) : g == 0) : ((head_per_wave || wave == 0) && g == 0);
 
   // ---- where a finished row goes ---------------------------------------------------------
   // Normally into its partial slot (fp32, merged by the second kernel). A launch in which every
@@ -349,6 +357,95 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
   };
 
   if (tall) {
+    if constexpr (TALLK == 16) {
+    constexpr int NP = D / 64;             // 16-byte K (and V) loads per thread per step
+    constexpr int PF = 3;                  // steps kept in flight per workgroup (a 4th costs the registers that let the operand
+                                           // reads of a step run ahead of its MFMAs: lone tall workgroups 6 % slower per step)
+    constexpr int RSK = D * 2 + 16;        // LDS row stride of a K tile (conflict-free 16-byte row reads)
+    constexpr int SHARED = kStepTokens * (RSK + RSV);    // one K + V stage
+    static_assert(2 * SHARED <= split_smem_bytes(D, 16), "LDS size");
+    const int nsteps_u = (ntok_u + kStepTokens - 1) / kStepTokens;
+    // ============ tall box, 16-row tile per wave: 32-token tiles shared through LDS ============
+    // Each step's K and V tile is fetched once per workgroup: thread t loads pieces t, t + 256 ..
+    // of the tile (16 lanes cover one 256-byte row), PF steps ahead, and drops them into one of
+    // two LDS stages; after a barrier every wave runs its own 16 rows against the stage.
+    u32x4 kst[PF][NP], vst[PF][NP];
+    int tok_in[NP];
+    unsigned koff[NP], voff[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      tok_in[i] = (i * kThreads + tid) / CPR;                 // token of the step, 0..31
+      const unsigned col = ((i * kThreads + tid) % CPR) * 16;
+      koff[i] = (unsigned)((tok_in[i] & 15) * kss) + col;
+      voff[i] = (unsigned)((tok_in[i] & 15) * vss) + col;
+    }
+    // Steps are fetched in order, so the half a wave reads next is tracked on the scalar unit
+    // (page of the chunk, 16-token slot in the page, byte offset of the slot) instead of being
+    // derived from the step number every time: a few scalar adds per half. Page strides are
+    // below 4 GiB (checked on the host): page id x stride is one 32 x 32 -> 64 bit multiply.
+    int f_page = 0, f_slot = 0;
+    unsigned f_koff = 0, f_voff = 0;
+    const unsigned ksp32 = (unsigned)ksp, vsp32 = (unsigned)vsp, k16 = (unsigned)(16 * kss), v16 = (unsigned)(16 * vss);
+    auto next_half = [&]() {
+      ++f_slot; f_koff += k16; f_voff += v16;
+      if (f_slot == hpp) { f_slot = 0; f_koff = 0; f_voff = 0; ++f_page; }
+    };
+    // D = 64: one load per step and thread, waves 2 and 3 read the step's second half
+    if (NP == 1 && __builtin_amdgcn_readfirstlane(wave >> 1)) next_half();
+    auto fetch = [&](int st, u32x4 (&kd)[NP], u32x4 (&vd)[NP]) {
+      if ((st + 1) * kStepTokens <= ntok_u) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const unsigned pg = (unsigned)__builtin_amdgcn_readlane(f_page < 64 ? pg0 : pg1, f_page & 63);
+          kd[i] = *(const u32x4*)(kbase + ((uint64_t)pg * ksp32 + f_koff) + koff[i]);
+          vd[i] = *(const u32x4*)(vbase + ((uint64_t)pg * vsp32 + f_voff) + voff[i]);
+          next_half();
+        }
+        if (NP == 1) next_half();
+      } else {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const unsigned col = ((i * kThreads + tid) % CPR) * 16;
+          kd[i] = *(const u32x4*)(lane_row(kbase, ksp, kss, st * kStepTokens + tok_in[i]) + col);
+          vd[i] = *(const u32x4*)(lane_row(vbase, vsp, vss, st * kStepTokens + tok_in[i]) + col);
+        }
+      }
+    };
+#pragma unroll
+    for (int s = 0; s < PF; ++s)
+      if (s < nsteps_u) fetch(s, kst[s], vst[s]);
+    load_q();
+    for (int st0 = 0; st0 < nsteps_u; st0 += PF) {
+#pragma unroll
+      for (int s = 0; s < PF; ++s) {
+        const int st = st0 + s;
+        if (st >= nsteps_u) break;
+        PAT_LDS char* stage = (PAT_LDS char*)smem + (st & 1) * SHARED;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const int tok_in = (i * kThreads + tid) / CPR;
+          const int col16 = ((i * kThreads + tid) % CPR) * 16;
+          *(PAT_LDS u32x4*)(stage + tok_in * RSK + col16) = kst[s][i];
+          *(PAT_LDS u32x4*)(stage + kStepTokens * RSK + tok_in * RSV + col16) = vst[s][i];
+        }
+        if (st + PF < nsteps_u) fetch(st + PF, kst[s], vst[s]);
+        __syncthreads();
+        if (has_rows)
+          attend([&](int a, int kk) { return *(const PAT_LDS vec8*)(stage + (a * 16 + n) * RSK + (kk * 32 + g * 8) * 2); },
+                 stage + kStepTokens * RSK, t_begin + st * kStepTokens, []() {});
+      }
+    }
+    l_run = sum_xor32(sum_xor16(l_run));
+    if (my_slot0 >= 0) {
+      const int64_t prow = (int64_t)my_slot0;
+      const float inv = 1.f / l_run;
+      float* dst = p.o_part + prow * D + g * 4;
+      T* o = direct ? row_out(my_slot0) + g * 4 : nullptr;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) put4(dst + db * 16, o + db * 16, acc_o[db] * inv);
+      if (g == 0) put_lse(prow, (m_run + __builtin_amdgcn_logf(l_run)) * 0.6931471805599453f);
+    }
+    } else {
     // ====================== tall box: 32-row tiles, K/V shared through LDS ======================
     // The chunk is walked in super-steps of 64 tokens. Thread t loads pieces t, t + 256 .. of a
     // super-step's K and V tiles (16 lanes cover one 256-byte row), PF2 super-steps ahead in
@@ -370,7 +467,7 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
     constexpr int RSV2 = D * 2 + 64;       // LDS row stride of a V tile (conflict-free transposed reads)
     constexpr int STAGE2 = SST * (RSK2 + RSV2);
     constexpr int TPR = kThreads / CPR;    // tokens one load round of the workgroup covers: 16 (D 128) or 32 (D 64)
-    static_assert(2 * STAGE2 <= split_smem_bytes(D), "LDS size");
+    static_assert(2 * STAGE2 <= split_smem_bytes(D, 32), "LDS size");
     static_assert(2 * (D / 8) * 64 * 16 <= 2 * STAGE2, "the exchange buffer of the epilogue fits the stages");
     const int nss_u = (ntok_u + SST - 1) / SST;
     const float sc_abs = __builtin_fabsf(p.scale_log2);
@@ -594,6 +691,7 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
         }
       if (h2 == 0) put_lse(prow, (mm + __builtin_amdgcn_logf(lsum)) * 0.6931471805599453f);
     }
+    }   // TALLK
   } else {
     // ====================== short box: KV steps split over the 4 waves ========================
     // Each wave keeps DEPTH of its steps in flight in a ring of register buffers: when a step has
@@ -717,24 +815,26 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D)) pat_split_kernel
   }
 }
 
-// Host launcher: picks the instance for (element type, head_dim).
+// Host launcher: picks the instance for (element type, head_dim, single-slot launch, form of the tall path).
 typedef void (*SplitFn)(const char*, int, int, const SplitParams);
-template <bool DIRECT>
+template <bool DIRECT, int TALLK>
 static SplitFn split_instance(bool bf16, int head_dim) {
-  if (bf16) return head_dim == 64 ? pat_split_kernel<__bf16, 64, DIRECT> : pat_split_kernel<__bf16, 128, DIRECT>;
-  return head_dim == 64 ? pat_split_kernel<_Float16, 64, DIRECT> : pat_split_kernel<_Float16, 128, DIRECT>;
+  if (bf16) return head_dim == 64 ? pat_split_kernel<__bf16, 64, DIRECT, TALLK> : pat_split_kernel<__bf16, 128, DIRECT, TALLK>;
+  return head_dim == 64 ? pat_split_kernel<_Float16, 64, DIRECT, TALLK> : pat_split_kernel<_Float16, 128, DIRECT, TALLK>;
 }
 
 hipError_t launch_split(bool bf16, int head_dim, hipStream_t stream, const SplitParams& params) {
-  SplitFn fn = params.direct ? split_instance<true>(bf16, head_dim) : split_instance<false>(bf16, head_dim);
-  const unsigned lds = (unsigned)split_smem_bytes(head_dim);
+  const bool t32 = params.tall_rows != 16;
+  SplitFn fn = params.direct ? (t32 ? split_instance<true, 32>(bf16, head_dim) : split_instance<true, 16>(bf16, head_dim))
+                             : (t32 ? split_instance<false, 32>(bf16, head_dim) : split_instance<false, 16>(bf16, head_dim));
+  const unsigned lds = (unsigned)split_smem_bytes(head_dim, t32 ? 32 : 16);
   // more dynamic LDS than the default limit of a kernel: raised once per instance and device
   {
     static std::mutex mutex;
-    static bool raised[64][8] = {{false}};
+    static bool raised[64][16] = {{false}};
     int dev = 0;
     if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-    const int inst = (bf16 ? 4 : 0) + (head_dim == 128 ? 2 : 0) + (params.direct ? 1 : 0);
+    const int inst = (t32 ? 8 : 0) + (bf16 ? 4 : 0) + (head_dim == 128 ? 2 : 0) + (params.direct ? 1 : 0);
     std::lock_guard<std::mutex> lock(mutex);
     if (dev >= 0 && dev < 64 && !raised[dev][inst]) {
       if (const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

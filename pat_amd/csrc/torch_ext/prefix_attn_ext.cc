@@ -1046,7 +1046,7 @@ PYBIND11_MODULE(_prefix_attn, m) {
           const pat_fwd_tuning& t = kv.second->tuning;
           if (kv.second->args.tuning == nullptr) out.emplace_back();
           else out.push_back({t.chunk_tokens, t.tall_chunk_tokens, t.head_per_wave_tokens, t.head_per_wave_long_tokens,
-                              t.head_per_wave_long_wgs, t.equalize_chunks, t.direct_out});
+                              t.head_per_wave_long_wgs, t.equalize_chunks, t.direct_out, t.tall_rows});
         }
         return out;
       })

@@ -576,6 +576,42 @@ def test_large_ragged_batch_all_launch_modes(heads, dtype, tuning):
     _assert_close("large ragged, a kv head per wave", out, lse, ref_out, ref_lse, dtype)
 
 
+@pytest.mark.parametrize("tall_rows", [16, 32])
+@pytest.mark.parametrize("name", ["c2", "c3", "c5a", "forest64", "tails"])
+def test_both_forms_of_the_tall_path(name, tall_rows, tuning):
+    # boxes of 17..64 rows run on 32-row tiles (32x32x16 MFMAs, 64-token super-steps) or on a 16-row
+    # tile per wave (16x16x32, 32-token steps); the launch picks one from its sizes, here each is forced
+    print(f"[case] tall path on {tall_rows}-row tiles: {name}", flush=True)
+    import ctypes as C
+    from pat_amd import _ctypes_launch, _lib
+    dev = _device()
+    if name == "forest64":      # head_dim 64, fp16, ragged forest with 17..64-row boxes and partial last steps
+        w = workloads.forest("forest64", 90, 3, 16, 4, 64, torch.float16, 11, root_range=(100, 1300),
+                             inner_range=(16, 400), leaf_range=(1, 120))
+    elif name == "tails":       # tall boxes whose length is no multiple of 64, 32 or 16 tokens, 17..40 rows
+        w = workloads.shared_prefix("tails", 10, 16 * 37, 1, 9, 32, 8, 128, torch.bfloat16, 5)
+    else:
+        w = workloads.make(name, seed=2)
+    tuning(tall_rows=tall_rows)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    lt = info.launch_tables()
+    L = _ctypes_launch.prepare(q, k, v, info.num_boxes_per_seq, lt["q_tables"], lt["block_tables"], lt["num_seqs_per_CTAs"],
+                               lt["CTA_ranks"], lt["kv_in_CTAs"], lt["MNWs"], info.max_boxes_per_seq, info.max_seqs_in_CTA,
+                               info.max_blocks_in_CTA, 1.0 / math.sqrt(w.head_dim), torch.empty_like(q), None,
+                               lt["slot_tables"], lt.get("flags"))
+    geo = _lib.FwdGeometry()
+    assert _lib.load().pat_fwd_geometry_of(C.byref(L.args), C.byref(geo)) == 0 and geo.tall_rows == tall_rows
+    assert any(m[0] > 16 for m in info.MNWs), "the case has no tall box"
+    out, lse = _run_tree(w, q, k, v)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close(f"{name}, {tall_rows}-row tiles", out, lse, ref_out, ref_lse, w.dtype)
+
+
 def test_strided_views_and_output_in_place():
     # vLLM hands in views: q/out are slices of larger buffers, K and V live in one stacked tensor
     print("[case] strided views", flush=True)
@@ -781,7 +817,7 @@ def test_autotuned_geometry_matches_oracle_and_is_remembered():
             if i == 0:
                 _assert_close("c2 drop-in call, tuned", out, lse, ref_out, ref_lse, w.dtype)
         chosen = info._launch_tunings
-        assert len(chosen) == 2 and chosen[0] == chosen[1] and len(chosen[0]) == 7
+        assert len(chosen) == 2 and chosen[0] == chosen[1] and len(chosen[0]) == 8
     finally:
         _prefix_attn.set_autotune(was)
 

@@ -112,9 +112,11 @@ def test_geometry_and_workspace_are_consistent():
     g = _lib.FwdGeometry()
     assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
     assert g.chunk_tokens % 32 == 0 and g.tall_chunk_tokens % 32 == 0
-    # 4 tall boxes x 8 kv heads are cut until there are about three workgroups per eight CUs: 3 pieces;
-    # the 64 boxes of up to 512 tokens run a kv head per wave on 256-token pieces (2 per box, 2 head groups)
-    per_box = [3, 2]
+    # the launch waits for its 64 boxes of up to 512 tokens, not for its 4 tall boxes: those run the
+    # 16-row form (3 workgroups per CU) and are cut until there is a tall workgroup per two CUs: 4 pieces;
+    # the 64 boxes run a kv head per wave on 256-token pieces (2 per box, 2 head groups)
+    assert g.tall_rows == 16
+    per_box = [4, 2]
     assert -(-128 * 16 // g.tall_chunk_tokens) == per_box[0]
     assert g.chunks_per_rank == max(per_box)
     assert g.num_slots == g.chunks_per_rank * 2
@@ -225,6 +227,13 @@ def test_tuning_round_trip(tuning):
     assert (t.chunk_tokens, t.tall_chunk_tokens, t.head_per_wave_tokens, t.direct_out) == (256, 0, -1, 0)
     g = _lib.FwdGeometry()
     assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0 and g.chunk_tokens == 256
+    # the form of the tall path: chosen per launch unless set
+    for rows in (32, 16):
+        tuning(tall_rows=rows)
+        assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0 and g.tall_rows == rows
+    tuning(tall_rows=32)
+    assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0
+    assert -(-128 * 16 // g.tall_chunk_tokens) == 3      # 32-row tiles: about three tall workgroups per eight CUs
 
 
 def test_tree_handles_and_errors():
