@@ -100,7 +100,9 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
     made_o, keep_o = launches(oblivious, None)
     t_obl = timed(made_o)
     unique_bytes = w.unique_kv_bytes
-    return {"tree": spec, "heads": heads, "kv_heads": kv_heads, "batch": w.batch, "unique_kv_mb": unique_bytes / 1e6,
+    geo = _lib.FwdGeometry()
+    _lib.check(lib.pat_fwd_geometry_of(C.byref(made_a[0].args), C.byref(geo)))
+    return {"workgroups": int(geo.num_workgroups), "tall_rows": int(geo.tall_rows), "tree": spec, "heads": heads, "kv_heads": kv_heads, "batch": w.batch, "unique_kv_mb": unique_bytes / 1e6,
             "total_kv_mb": w.kv_bytes(w.total_tokens) / 1e6, "pat_us": t_aware, "oblivious_us": t_obl,
             "speedup": t_obl / t_aware, "unique_kv_gbs": unique_bytes / t_aware / 1e3, "kv_copies": copies}
 
@@ -118,14 +120,14 @@ def main() -> None:
         sys.exit("bench_trees needs an AMD GPU")
     trees = TREES if a.trees == ["all"] else a.trees
     rows = []
-    print(f"{'tree':48s} {'heads':>6s} {'batch':>5s} {'uniq MB':>8s} {'PAT us':>9s} {'obliv us':>9s} {'x':>6s} {'uniq GB/s':>9s}")
+    print(f"{'tree':48s} {'heads':>6s} {'batch':>5s} {'uniq MB':>8s} {'PAT us':>9s} {'obliv us':>9s} {'x':>6s} {'uniq GB/s':>9s} {'wgs':>6s} {'tall':>4s}")
     for spec in trees:
         for pair in a.heads:
             hq, hkv = (int(x) for x in pair.split())
             r = run_case(spec, hq, hkv, a.iters, a.warmup, int(a.cache_budget_gib * 2**30))
             rows.append(r)
             print(f"{spec:48s} {hq:3d}/{hkv:<2d} {r['batch']:5d} {r['unique_kv_mb']:8.1f} {r['pat_us']:9.1f} "
-                  f"{r['oblivious_us']:9.1f} {r['speedup']:6.2f} {r['unique_kv_gbs']:9.0f}", flush=True)
+                  f"{r['oblivious_us']:9.1f} {r['speedup']:6.2f} {r['unique_kv_gbs']:9.0f} {r['workgroups']:6d} {r['tall_rows']:4d}", flush=True)
             torch.cuda.empty_cache()
     if a.json:
         with open(a.json, "w") as f:

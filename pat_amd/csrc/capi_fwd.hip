@@ -172,7 +172,8 @@ int check_args(const pat_fwd_args* a) {
 //    write 16..32 KB of partial output per workgroup: their chunk is at least 256 tokens, and
 //    longer when they alone would still fill the device.
 // pat_fwd_tuning.chunk_tokens / tall_chunk_tokens override the two sizes (tuning aid).
-int plan_geometry(const pat_fwd_args* a, Geometry* g) {
+// (tall_rows: the form of the tall path the geometry is made for, 16 or 32)
+int plan_geometry_for(const pat_fwd_args* a, Geometry* g, int tall_rows) {
   const pat_fwd_tuning tune = a->tuning != nullptr ? *a->tuning : tuning();
   const int page = a->page_size;
   const int64_t unit = (int64_t)page * kStepTokens / gcd64(page, kStepTokens);  // lcm(page, 32)
@@ -183,21 +184,6 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   for (int i = 0; i < a->num_buckets; ++i) {
     const int64_t w = (int64_t)a->buckets[i].max_blocks * page * a->buckets[i].num_boxes * a->kv_heads;
     if (row_tiles(a->buckets[i].mnw[0]) == 1) work += w;
-  }
-  // Which form of the tall path (boxes of 17..64 rows): 32-row tiles walk a tall box faster and cost a
-  // resident workgroup per CU at head_dim 128; they pay where the launch waits for its tall boxes.
-  // Estimated from sizes: a tall workgroup takes ~1.25 us per 64 tokens, the <= 16-row boxes stream at
-  // ~5.8 TB/s, ragged buckets (no PAT_BUCKET_EVEN hint) hold ~0.6 of their widest box on average.
-  int tall_rows = tune.tall_rows == 16 || tune.tall_rows == 32 ? tune.tall_rows : 0;
-  if (tall_rows == 0) {
-    double tall_us = 0., short_us = 0.;
-    for (int i = 0; i < a->num_buckets; ++i) {
-      const pat_fwd_bucket& b = a->buckets[i];
-      const double token_heads = (double)b.max_blocks * page * b.num_boxes * a->kv_heads;
-      if (row_tiles(b.mnw[0]) > 1) tall_us += token_heads / 64. * 1.25 / kNumCUs;
-      else short_us += token_heads * ((b.flags & PAT_BUCKET_EVEN) ? 1.0 : 0.6) * a->head_dim * 4. / 5.8e6;
-    }
-    tall_rows = tall_us > 0. && tall_us >= short_us ? 32 : 16;
   }
   g->tall_rows = tall_rows;
   const int64_t resident = (int64_t)resident_wgs_per_cu(a->head_dim, tall_rows) * kNumCUs;
@@ -386,6 +372,38 @@ int plan_geometry(const pat_fwd_args* a, Geometry* g) {
   if ((int64_t)a->batch * a->heads * g->num_slots >= ((int64_t)1 << 31))
     return fail(PAT_ERR_INVALID, "batch * heads * partial slots must stay below 2^31");
   return PAT_OK;
+}
+
+// Which form of the tall path (boxes of 17..64 rows)? 32-row tiles walk a tall box faster and cost a
+// resident workgroup per CU at head_dim 128. They are taken when that costs nothing - the whole launch
+// is resident at two workgroups per CU anyway - or when the launch waits for its tall boxes: those are
+// long (1024 tokens or more: short ones are mostly prologue and epilogue in either form) and, estimated
+// from sizes, take at least as long as the <= 16-row boxes (a tall workgroup ~1.25 us per 64 tokens;
+// the others stream at ~5.8 TB/s; ragged buckets, without the PAT_BUCKET_EVEN hint, hold ~0.6 of their
+// widest box on average). Measured (us per call, 16 / 32 rows): c2 26.1 / 25.7, c3 70.9 / 72.7,
+// c5a 70.6 / 67.4; sweep trees with 512-1024 short leaves 5-14 % faster on 16, `1,1024_2048,32` 3 % on 32.
+int plan_geometry(const pat_fwd_args* a, Geometry* g) {
+  const pat_fwd_tuning tune = a->tuning != nullptr ? *a->tuning : tuning();
+  if (tune.tall_rows == 16 || tune.tall_rows == 32) return plan_geometry_for(a, g, tune.tall_rows);
+  double tall_us = 0., short_us = 0.;
+  int64_t widest_tall = 0;
+  for (int i = 0; i < a->num_buckets; ++i) {
+    const pat_fwd_bucket& b = a->buckets[i];
+    if (b.num_boxes <= 0) continue;
+    const double token_heads = (double)b.max_blocks * a->page_size * b.num_boxes * a->kv_heads;
+    if (row_tiles(b.mnw[0]) > 1) {
+      tall_us += token_heads / 64. * 1.25 / kNumCUs;
+      widest_tall = std::max<int64_t>(widest_tall, (int64_t)b.max_blocks * a->page_size);
+    } else {
+      short_us += token_heads * ((b.flags & PAT_BUCKET_EVEN) ? 1.0 : 0.6) * a->head_dim * 4. / 5.8e6;
+    }
+  }
+  if (widest_tall == 0) return plan_geometry_for(a, g, 16);   // no tall box: the form with more resident workgroups
+  if (int rc = plan_geometry_for(a, g, 32)) return rc;
+  if (g->total_wgs <= (int64_t)resident_wgs_per_cu(a->head_dim, 32) * kNumCUs) return PAT_OK;
+  if (widest_tall >= 1024 && tall_us >= short_us) return PAT_OK;
+  *g = Geometry();
+  return plan_geometry_for(a, g, 16);
 }
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }

@@ -112,11 +112,11 @@ def test_geometry_and_workspace_are_consistent():
     g = _lib.FwdGeometry()
     assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0
     assert g.chunk_tokens % 32 == 0 and g.tall_chunk_tokens % 32 == 0
-    # the launch waits for its 64 boxes of up to 512 tokens, not for its 4 tall boxes: those run the
-    # 16-row form (3 workgroups per CU) and are cut until there is a tall workgroup per two CUs: 4 pieces;
-    # the 64 boxes run a kv head per wave on 256-token pieces (2 per box, 2 head groups)
-    assert g.tall_rows == 16
-    per_box = [4, 2]
+    # the whole launch is resident at two workgroups per CU: the tall boxes take the 32-row form and are cut
+    # until there are about three tall workgroups per eight CUs: 3 pieces; the 64 boxes of up to 512 tokens
+    # run a kv head per wave on 256-token pieces (2 per box, 2 head groups)
+    assert g.tall_rows == 32
+    per_box = [3, 2]
     assert -(-128 * 16 // g.tall_chunk_tokens) == per_box[0]
     assert g.chunks_per_rank == max(per_box)
     assert g.num_slots == g.chunks_per_rank * 2
@@ -231,9 +231,9 @@ def test_tuning_round_trip(tuning):
     for rows in (32, 16):
         tuning(tall_rows=rows)
         assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0 and g.tall_rows == rows
-    tuning(tall_rows=32)
+    tuning(tall_rows=16)
     assert lib.pat_fwd_geometry_of(C.byref(_args()), C.byref(g)) == 0
-    assert -(-128 * 16 // g.tall_chunk_tokens) == 3      # 32-row tiles: about three tall workgroups per eight CUs
+    assert -(-128 * 16 // g.tall_chunk_tokens) == 4      # the 16-row form: a tall workgroup per two CUs
 
 
 def test_tree_handles_and_errors():
