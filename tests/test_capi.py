@@ -271,3 +271,25 @@ def test_baseline_workspace_and_errors_without_a_gpu():
     assert "max_blocks" in _lib.last_error()
     a.max_blocks, a.kv_heads = 256, 5
     assert lib.pat_paged_decode_baseline_workspace_bytes(C.byref(a), C.byref(need)) == _lib.PAT_ERR_INVALID
+
+
+def test_form_of_the_tall_path_follows_the_launch():
+    """32-row tiles when the whole launch is resident at two workgroups per CU or its long tall boxes
+    outweigh the short ones; the 16-row form (a third resident workgroup per CU) otherwise."""
+    lib = _lib.load()
+    g = _lib.FwdGeometry()
+
+    def form(tall_boxes, tall_blocks, short_boxes, short_blocks, batch):
+        a = _args(batch=batch)
+        b = a._keep
+        b[0].num_boxes, b[0].max_blocks, b[0].block_table_stride = tall_boxes, tall_blocks, tall_blocks
+        b[1].num_boxes, b[1].max_blocks, b[1].block_table_stride = short_boxes, short_blocks, short_blocks
+        a.max_blocks_in_box = max(tall_blocks, short_blocks)
+        assert lib.pat_fwd_geometry_of(C.byref(a), C.byref(g)) == 0, _lib.last_error()
+        return g.tall_rows, g.num_workgroups
+
+    assert form(4, 128, 64, 32, 64)[0] == 32            # the headline batch: everything resident at once
+    assert form(16, 64, 128, 64, 128)[0] == 16          # a 3-level tree: 1024-token leaves outweigh the tall boxes
+    assert form(24, 171, 32, 128, 32)[0] == 32          # a 16k prefix in 2736-token tall boxes over 2048-token suffixes
+    assert form(128, 8, 1024, 2, 1024)[0] == 16         # many short tall boxes over a thousand 32-token leaves
+    assert form(0, 128, 512, 64, 512)[0] == 16          # no tall box at all
