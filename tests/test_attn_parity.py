@@ -736,11 +736,12 @@ def test_validation_errors_on_gpu_tensors():
                                  0.125, out[..., :32].contiguous())
 
 
-def test_randomized_workloads_fixed_seed():
+def test_randomized_workloads_fixed_seed(tuning):
     # 120 workloads drawn from a fixed seed: independent requests, one shared prefix, three-level trees
     # and irregular forests over 8 head configurations, both head dims and element types; small ones
     # (the oracle runs on the CPU). Batches without sharing of 27 requests or more take the
-    # single-slot route, the rest every other route the launch geometry knows.
+    # single-slot route, the rest every other route the launch geometry knows. The form of the tall
+    # path is the launch's own choice in every third case and forced to 16 / 32 rows in the others.
     import numpy as np
     dev = _device()
     rng = np.random.default_rng(20240607)
@@ -765,7 +766,8 @@ def test_randomized_workloads_fixed_seed():
                                  root_range=(64, 1500), inner_range=(16, 300), leaf_range=(1, 200))
         if w.kv_bytes(w.total_tokens) > 1.5e8:
             continue
-        print(f"[case] random {done}: kind {kind} batch {w.batch} heads {h}/{hk} d {d} {dtype} seed {seed}", flush=True)
+        print(f"[case] random {done}: kind {kind} batch {w.batch} heads {h}/{hk} d {d} {dtype} seed {seed} tall form {(0, 16, 32)[done % 3]}", flush=True)
+        tuning(tall_rows=(0, 16, 32)[done % 3])
         q, k, v = w.tensors(dev)
         out, lse = _run_tree(w, q, k, v)
         ref_out, ref_lse = _oracle(w, q, k, v)
