@@ -68,6 +68,16 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
                  num_seqs_per_CTAs=lt["num_seqs_per_CTAs"], CTA_ranks=lt["CTA_ranks"], kv_in_CTAs=lt["kv_in_CTAs"],
                  MNW=lt["MNWs"], max_split_per_seq=info.max_split_per_seq, max_seqs_in_CTA=info.max_seqs_in_CTA,
                  max_blocks_in_CTA=info.max_blocks_in_CTA, bucket_flags=lt.get("flags"))
+    aware_slots = lt["slot_tables"]
+    whole = info.whole_sequence_tables()
+    if whole is not None:
+        # a small batch of short requests: the drop-in call launches one work item per request (one kernel)
+        aware = dict(num_split_per_seq=whole["num_split_per_seq"], query_tables=whole["q_tables"],
+                     block_tables=whole["block_tables"], num_seqs_per_CTAs=whole["num_seqs_per_CTAs"],
+                     CTA_ranks=whole["CTA_ranks"], kv_in_CTAs=whole["kv_in_CTAs"], MNW=whole["MNWs"],
+                     max_split_per_seq=whole["max_split_per_seq"], max_seqs_in_CTA=whole["max_seqs_in_CTA"],
+                     max_blocks_in_CTA=whole["max_blocks_in_CTA"], bucket_flags=None)
+        aware_slots = None
     oblivious = workloads.oblivious_plan(w, dev)
 
     def launches(plan, slots):
@@ -95,14 +105,14 @@ def run_case(spec: str, heads: int, kv_heads: int, iters: int, warmup: int, budg
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / iters * 1e3
 
-    made_a, keep_a = launches(aware, lt["slot_tables"])
+    made_a, keep_a = launches(aware, aware_slots)
     t_aware = timed(made_a)
     made_o, keep_o = launches(oblivious, None)
     t_obl = timed(made_o)
     unique_bytes = w.unique_kv_bytes
     geo = _lib.FwdGeometry()
     _lib.check(lib.pat_fwd_geometry_of(C.byref(made_a[0].args), C.byref(geo)))
-    return {"workgroups": int(geo.num_workgroups), "tall_rows": int(geo.tall_rows), "tree": spec, "heads": heads, "kv_heads": kv_heads, "batch": w.batch, "unique_kv_mb": unique_bytes / 1e6,
+    return {"workgroups": int(geo.num_workgroups), "tall_rows": int(geo.tall_rows), "whole_sequences": whole is not None, "tree": spec, "heads": heads, "kv_heads": kv_heads, "batch": w.batch, "unique_kv_mb": unique_bytes / 1e6,
             "total_kv_mb": w.kv_bytes(w.total_tokens) / 1e6, "pat_us": t_aware, "oblivious_us": t_obl,
             "speedup": t_obl / t_aware, "unique_kv_gbs": unique_bytes / t_aware / 1e3, "kv_copies": copies}
 

@@ -440,7 +440,7 @@ struct KernelInfo {
   // the block rows [batch, ws_width].
   bool whole_seqs = false;
   int64_t ws_offset = 0;
-  int ws_batch = 0, ws_width = 0, ws_tile = 16;
+  int ws_batch = 0, ws_width = 0, ws_tile = 16, ws_longest_allowed = 0;
   TensorList ws_q_table, ws_block_table, ws_num_seqs, ws_rank, ws_kv;
   std::vector<std::vector<int>> ws_mnw;
   at::Tensor ws_num_split;
@@ -562,6 +562,7 @@ struct KernelInfo {
     d["CTA_ranks"] = ws_rank; d["kv_in_CTAs"] = ws_kv; d["MNWs"] = ws_mnw;
     d["num_split_per_seq"] = ws_num_split; d["max_split_per_seq"] = 1; d["max_seqs_in_CTA"] = 1;
     d["max_blocks_in_CTA"] = ws_width;
+    d["longest_allowed"] = ws_longest_allowed;   // a request that outgrows this takes the batch back to the tree's plan
     return d;
   }
 
@@ -594,15 +595,20 @@ struct TreeHandle {
 
 // Is a batch better served by one work item per request than by its prefix-aware plan? Yes when the
 // whole launch is a few microseconds of latency anyway: every request short enough for one workgroup
-// to walk in a few steps per wave, at most two workgroups per CU, and so little KV in total that
+// to walk in a few steps per wave, everything resident at once, and so little KV in total that
 // re-reading shared pages (from L2) costs less than the merge kernel's launch and round trips.
-bool whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page) {
+// Measured (us per call, plan / one item per request): 8 requests of 288 tokens 6.7 / 5.9; 32 x 192:
+// 10.4 / 6.5; 64 x 192: 10.4 / 8.3; 32 x 384: 13.7 / 9.3; 16 x 512: 13.6 / 10.0; 8 x 768: 10.6-13.1 /
+// 9.4-10.0; 8 x 1088: 11.2 / 11.1. Without query-head groups (a kv head per query head: no 17..64-row
+// boxes in the plan) the plan keeps up sooner: 12 x 576: 8.1 / 9.3, so the bound is 384 tokens there.
+int whole_sequence_limit(int hratio) { return hratio >= 2 ? 768 : 384; }
+bool whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page, int hratio) {
   if (lens.empty() || kv_heads <= 0) return false;
   int64_t total = 0, longest = 0;
   for (int32_t n : lens) { total += n; longest = std::max<int64_t>(longest, n); }
   const int64_t bytes = total * kv_heads * 128 * 2 * 2;   // (at head_dim 128; the planner does not know it)
-  return longest > 0 && longest <= 512 && (int64_t)lens.size() * kv_heads <= 512 && bytes <= (int64_t)16 << 20 &&
-         page > 0;
+  return longest > 0 && longest <= whole_sequence_limit(hratio) && (int64_t)lens.size() * kv_heads <= 512 &&
+         bytes <= (int64_t)64 << 20 && page > 0;
 }
 
 struct PrefixTreeCPP {
@@ -760,7 +766,7 @@ struct PrefixTreeCPP {
       int64_t total = std::max<int64_t>(fresh->layout.total, 1);
       const int64_t nb = (int64_t)batch_lens.size();
       if (hratio >= 1 && hratio <= 16 && fresh->layout.batch == nb && batch_table.defined() && batch_table.size(0) == nb &&
-          whole_sequences_pay(batch_lens, kv_head, block_size)) {
+          whole_sequences_pay(batch_lens, kv_head, block_size, hratio)) {
         int64_t longest = 0;
         for (int32_t n : batch_lens) longest = std::max<int64_t>(longest, n);
         fresh->whole_seqs = true;
@@ -768,6 +774,7 @@ struct PrefixTreeCPP {
         // (8 spare columns: room for in-place growth between decode steps)
         fresh->ws_width = (int)std::min<int64_t>(batch_table.size(1), (longest + block_size - 1) / block_size + 8);
         fresh->ws_tile = 16;
+        fresh->ws_longest_allowed = whole_sequence_limit(hratio);
         fresh->ws_offset = total;
         total += 4 * nb + nb * fresh->ws_width;
       }

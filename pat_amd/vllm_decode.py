@@ -184,7 +184,7 @@ class DecodePlan:
         whole = info.whole_sequence_tables()
         if whole is not None:
             width = whole["block_tables"][0].shape[1]
-            if any(n_old % bs == 0 and n_old // bs >= width for n_old in old) or max(self.seq_lens) > 512:
+            if any(n_old % bs == 0 and n_old // bs >= width for n_old in old) or max(self.seq_lens) > whole["longest_allowed"]:
                 self._replan(table_cpu)
                 return False
         self._tail_kv += 1
