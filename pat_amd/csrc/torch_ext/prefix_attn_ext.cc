@@ -602,13 +602,48 @@ struct TreeHandle {
 // 9.4-10.0; 8 x 1088: 11.2 / 11.1. Without query-head groups (a kv head per query head: no 17..64-row
 // boxes in the plan) the plan keeps up sooner: 12 x 576: 8.1 / 9.3, so the bound is 384 tokens there.
 int whole_sequence_limit(int hratio) { return hratio >= 2 ? 768 : 384; }
-bool whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page, int hratio) {
-  if (lens.empty() || kv_heads <= 0) return false;
+// Beyond those small batches, the same launch serves any batch whose sharing saves little: the plan
+// reads every shared page once and pays for it with a second kernel, partial rows and the slower steps of
+// its 17..64-row boxes; one work item per request reads a shared page once per request that holds it,
+// from L2 after the first time. Both launches were timed on 1-level trees of 2..128 requests with
+// 256..16384 shared and 32..1024 private tokens at 32/32, 16/2, 32/8 and 64/8 heads, and on the reference's
+// tree sweep (benchmark/run_kernel_bench.sh:5-33); least squares with non-negative coefficients gives, in
+// us per call with U = MB of K and V the tree's nodes hold, S = MB that sharing saves (the same counted
+// once per request, minus U), rows = batch x query heads:
+//     one item per request  6.5 + 1.9 [a second kernel: see below] + 0.165 U + 0.070 S
+//     the plan              9.4 + 0.179 U + 0.002 S x (query heads per kv head) + 0.39 rows / 1000
+// (mean error 6 % and 10 %). One item per request is launched when its estimate is the lower one (with the
+// plan's constant at 9.8: that decides more of the close cases right) and S is below 200 MB (the measured
+// range of close calls; beyond it the plan won every case). Over the 356 measured cases the choice is
+// within 3 % of the faster launch in 329 (always the plan: 274) and at worst 19 % slower (always the plan:
+// 66 %); e.g. plan / one item per request: 64 x (256 + 32) tokens at 64/8
+// heads 13.4 / 10.8 us, 8 x (1024 + 1024) at 32/8 16.6 / 14.6, 128 x (256 + 32) at 16/2 13.0 / 7.9, against
+// 128 x (256 + 32) at 32/8 15.2 / 17.9, 4 x (4096 + 32) 13.3 / 15.3. No tree of the reference's sweep changes.
+// A request walked by one workgroup needs no second kernel: up to 512 tokens, or up to 2048 when the batch
+// has a box per CU (requests x kv heads >= 256); the launch cuts longer ones into pieces and merges them.
+constexpr double kWholeSavedMaxMB = 200.;
+// Returns the longest request the one-item-per-request launch stays right for (0: launch the plan).
+// unique_tokens: tokens held by the tree's nodes; shared: some request sits in two boxes of the plan.
+int whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page, int hratio, int64_t unique_tokens,
+                        bool shared) {
+  if (lens.empty() || kv_heads <= 0 || page <= 0) return 0;
   int64_t total = 0, longest = 0;
   for (int32_t n : lens) { total += n; longest = std::max<int64_t>(longest, n); }
-  const int64_t bytes = total * kv_heads * 128 * 2 * 2;   // (at head_dim 128; the planner does not know it)
-  return longest > 0 && longest <= whole_sequence_limit(hratio) && (int64_t)lens.size() * kv_heads <= 512 &&
-         bytes <= (int64_t)64 << 20 && page > 0;
+  if (longest <= 0) return 0;
+  const int64_t token_bytes = (int64_t)kv_heads * 128 * 2 * 2;   // (at head_dim 128; the planner does not know it)
+  int small = 0;
+  if (longest <= whole_sequence_limit(hratio) && (int64_t)lens.size() * kv_heads <= 512 && total * token_bytes <= (int64_t)64 << 20)
+    small = whole_sequence_limit(hratio);
+  if (!shared || unique_tokens <= 0 || unique_tokens > total) return small;   // nothing to merge in the plan either
+  const double unique_mb = (double)(unique_tokens * token_bytes) / 1e6;
+  const double saved_mb = (double)((total - unique_tokens) * token_bytes) / 1e6;
+  if (saved_mb >= kWholeSavedMaxMB) return small;
+  const double rows = (double)lens.size() * kv_heads * hratio;
+  const double plan_us = 9.8 + 0.179 * unique_mb + 0.002 * saved_mb * hratio + 0.39 * rows / 1000.;
+  const double whole_us = 6.5 + 0.165 * unique_mb + 0.070 * saved_mb;
+  if (whole_us + 1.9 < plan_us) return INT32_MAX;
+  const int64_t one_kernel = (int64_t)lens.size() * kv_heads >= 256 ? 2048 : 512;
+  return whole_us < plan_us && longest <= one_kernel ? std::max(small, (int)one_kernel) : small;
 }
 
 struct PrefixTreeCPP {
@@ -765,8 +800,17 @@ struct PrefixTreeCPP {
     if (rc_flat == PAT_OK) {
       int64_t total = std::max<int64_t>(fresh->layout.total, 1);
       const int64_t nb = (int64_t)batch_lens.size();
-      if (hratio >= 1 && hratio <= 16 && fresh->layout.batch == nb && batch_table.defined() && batch_table.size(0) == nb &&
-          whole_sequences_pay(batch_lens, kv_head, block_size, hratio)) {
+      int ws_allowed = 0;
+      if (hratio >= 1 && hratio <= 16 && fresh->layout.batch == nb && batch_table.defined() && batch_table.size(0) == nb) {
+        int64_t unique = 0;
+        const int n_nodes = pat_tree_num_nodes(native->h);
+        for (int i = 0; i < n_nodes; ++i) {
+          pat_node_view node;
+          if (pat_tree_node(native->h, i, &node) == PAT_OK && node.parent >= -1) unique += node.num_tokens;
+        }
+        ws_allowed = whole_sequences_pay(batch_lens, kv_head, block_size, hratio, unique, fresh->layout.max_split_per_seq > 1);
+      }
+      if (ws_allowed > 0) {
         int64_t longest = 0;
         for (int32_t n : batch_lens) longest = std::max<int64_t>(longest, n);
         fresh->whole_seqs = true;
@@ -774,7 +818,7 @@ struct PrefixTreeCPP {
         // (8 spare columns: room for in-place growth between decode steps)
         fresh->ws_width = (int)std::min<int64_t>(batch_table.size(1), (longest + block_size - 1) / block_size + 8);
         fresh->ws_tile = 16;
-        fresh->ws_longest_allowed = whole_sequence_limit(hratio);
+        fresh->ws_longest_allowed = ws_allowed;
         fresh->ws_offset = total;
         total += 4 * nb + nb * fresh->ws_width;
       }

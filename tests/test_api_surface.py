@@ -173,3 +173,47 @@ def test_plan_tensors_keep_version_counters_under_inference_mode():
         tree.kernel_info.kv_in_CTAs[0][0] += 1      # a view of the one buffer
         assert flat._version > before
     assert not tree.kernel_info.kv_in_CTAs[0].is_inference()
+
+
+def _packed(spec: str, heads: int, kv_heads: int, page: int = 32):
+    import random
+    from pat_amd import PrefixTreeCPP, generate_tree_seqs
+    random.seed(0)
+    group, _ = generate_tree_seqs(spec, page)
+    rows = group.get_block_ids()
+    width = max(len(r) for r in rows)
+    table = torch.zeros(len(rows), width, dtype=torch.int32)
+    for i, r in enumerate(rows):
+        table[i, :len(r)] = torch.tensor(r, dtype=torch.int32)
+    tree = PrefixTreeCPP(page)
+    tree.build_radix_tree(list(group.seqlens), table)
+    tree.pack_schedule(None, heads // kv_heads, kv_heads)
+    return tree.kernel_info, list(group.seqlens), rows
+
+
+def test_one_work_item_per_request_where_sharing_saves_little():
+    """The planner hands out the one-work-item-per-request tables (the launch the drop-in call then
+    makes) for batches whose shared pages are cheaper to re-read from L2 than the plan's second kernel
+    and partial rows are to pay, and for those only; sizes are of measured cases (plan / one item per
+    request, us per call): 64 x (256 + 32) tokens at 64/8 heads 13.4 / 10.8, 8 x (1024 + 1024) at 32/8
+    16.6 / 14.6, 128 x (256 + 32) at 16/2 13.0 / 7.9; 128 x (256 + 32) at 32/8 15.2 / 17.9,
+    4 x (4096 + 32) at 32/8 13.3 / 15.3, 64 x (2048 + 32) at 32/8 15.8 / 25.4."""
+    for spec, heads, kv_heads, expect in (("1,64_256,32", 64, 8, 2048), ("1,8_1024,1024", 32, 8, 2**31 - 1),
+                                          ("1,128_256,32", 16, 2, 2**31 - 1), ("1,128_256,32", 32, 8, None),
+                                          ("1,4_4096,32", 32, 8, None), ("1,64_1024,32", 32, 8, None),
+                                          ("1,1024_2048,32", 64, 8, None)):
+        info, lens, rows = _packed(spec, heads, kv_heads)
+        whole = info.whole_sequence_tables()
+        assert (whole is not None) == (expect is not None), spec
+        if whole is None:
+            continue
+        assert whole["longest_allowed"] == expect, spec
+        assert whole["max_split_per_seq"] == 1 and whole["MNWs"] == [[16, 128, 1]]
+        assert whole["kv_in_CTAs"][0].tolist() == lens
+        assert whole["q_tables"][0][:, 0].tolist() == list(range(len(lens)))
+        assert whole["block_tables"][0].shape[1] == max(len(r) for r in rows)     # (the caller's table has no spare columns)
+        for i, r in enumerate(rows):
+            assert whole["block_tables"][0][i, :len(r)].tolist() == r
+    # no request in two boxes: the plan has nothing to merge either, and is launched as it is
+    info, _, _ = _packed("600_64", 32, 8)
+    assert info.max_split_per_seq == 1 and info.whole_sequence_tables() is None

@@ -1140,3 +1140,34 @@ def test_small_batch_is_launched_as_whole_sequences():
     t2.build_radix_tree(big.seq_lens, big.padded_table())
     t2.pack_schedule(None, big.heads // big.kv_heads, big.kv_heads)
     assert t2.kernel_info.whole_sequence_tables() is None
+
+
+@pytest.mark.parametrize("spec,heads,kernels", [("1,8_1024,1024", (32, 8), 2), ("1,64_256,32", (64, 8), 1),
+                                                ("1,128_256,32", (16, 2), 1), ("1,4,8_512,256,704", (32, 8), 2)])
+def test_little_sharing_is_launched_as_whole_sequences(spec, heads, kernels):
+    # batches whose sharing saves less than the plan's second kernel costs: the tree form launches one
+    # work item per request - cut into pieces and merged when requests are long (a workspace then),
+    # one kernel when they are short - and equals the oracle
+    print(f"[case] little sharing: {spec} heads {heads}: one work item per request", flush=True)
+    import random
+    from pat_amd import generate_tree_seqs
+    dev = _device()
+    random.seed(5)
+    group, nblk = generate_tree_seqs(spec, 32)
+    w = workloads.Workload(spec, heads[0], heads[1], 128, torch.float16, 32, group.seqlens, group.get_block_ids(),
+                           nblk, 0, 4)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    whole = info.whole_sequence_tables()
+    assert whole is not None and info.max_split_per_seq >= 2
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    assert (info._launch_workspace_bytes == [0]) == (kernels == 1)
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("whole sequences " + spec, out, lse, ref_out, ref_lse, w.dtype)

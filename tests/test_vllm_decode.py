@@ -130,11 +130,26 @@ def _few_long_many_short():
     return workloads.Workload("wide-head", 8, 8, 64, torch.float16, 16, lens, rows, nxt, sum(lens), 0)
 
 
-@pytest.mark.parametrize("case", ["c1", "wide-head"])
+def _little_sharing():
+    """8 requests of 1023..1024 tokens over a 512-token shared prefix, 8/8 heads: longer than the
+    small-batch form goes, and sharing saves too little for the plan's second kernel, so the batch is
+    launched one work item per request (cut into pieces)."""
+    shared = list(range(32))
+    lens, rows, nxt = [], [], 32
+    for i in range(8):
+        n = 1024 - (i % 2)                    # even requests end on a page boundary: they grow at step 1
+        nb = -(-n // 16)
+        rows.append(shared + list(range(nxt, nxt + nb - 32)))
+        nxt += nb - 32
+        lens.append(n)
+    return workloads.Workload("little-sharing", 8, 8, 64, torch.float16, 16, lens, rows, nxt, 512 + sum(n - 512 for n in lens), 0)
+
+
+@pytest.mark.parametrize("case", ["c1", "wide-head", "little-sharing"])
 def test_advance_step_keeps_the_plan_right_on_cpu(case):
     """After every in-place advance the plan, executed item by item by the oracle, gives dense
     attention over the grown requests (c1: 8 requests x 288 tokens, so step 1 crosses a page)."""
-    w = workloads.make("c1", seed=5) if case == "c1" else _few_long_many_short()
+    w = {"c1": lambda: workloads.make("c1", seed=5), "wide-head": _few_long_many_short, "little-sharing": _little_sharing}[case]()
     steps = 20
     spare = list(range(w.num_blocks, w.num_blocks + 640))
     width = w.padded_table().shape[1] + 2
@@ -165,17 +180,26 @@ def test_advance_step_keeps_the_plan_right_on_cpu(case):
                     assert torch.equal(launch["block_tables"][lb], info.block_tables[b][order[lo:hi]][:, :lw])
                     assert (launch["kv_in_CTAs"][lb][:-1] >= launch["kv_in_CTAs"][lb][1:] - step).all()
             whole = info.whole_sequence_tables()    # small batches are launched a work item per request
-            assert (whole is not None) == (case == "c1")
+            assert (whole is not None) == (case in ("c1", "little-sharing"))
             if whole is not None:
                 assert whole["kv_in_CTAs"][0].tolist() == lens and whole["q_tables"][0][:, 0].tolist() == list(range(w.batch))
                 for i, r in enumerate(rows):
                     assert whole["block_tables"][0][i, :len(r)].tolist() == r
+            if case == "little-sharing":
+                # what is launched here are the one-item-per-request tables: those are executed (the plan of
+                # such a batch, few requests cut into many boxes, can hold one rank twice for a request, as
+                # the reference's does; the launch files its partial rows by box ordinal instead)
+                listed = {"q_tables": [whole["q_tables"][0].tolist()], "block_tables": [whole["block_tables"][0].tolist()],
+                          "num_seqs_per_CTAs": [whole["num_seqs_per_CTAs"][0].tolist()], "CTA_ranks": [whole["CTA_ranks"][0].tolist()],
+                          "kv_in_CTAs": [whole["kv_in_CTAs"][0].tolist()], "num_split_per_seq": whole["num_split_per_seq"].tolist()}
             out, lse = ao.run_plan_ref(listed, q, k, v)
             ref, ref_lse = ao.paged_attention_ref(q, k, v, rows, lens)
             assert (out - ref).abs().max().item() < 1e-5, step
             assert (lse - ref_lse).abs().max().item() < 1e-5, step
     assert in_place + plan.replans == steps
-    assert in_place >= steps - 2          # a full block row may force a fresh plan now and then
+    # a full block row may force a fresh plan now and then (more often where the scheduler has cut the
+    # requests into many boxes with block rows of their own)
+    assert in_place >= steps - (4 if case == "little-sharing" else 2)
 
 
 @pytest.mark.gpu
