@@ -20,6 +20,10 @@
 
 namespace pat {
 
+#ifndef PAT_MERGE_PAIRS_MIN
+#define PAT_MERGE_PAIRS_MIN 16384   // rows from which a half-wave takes a row (launches of up to 8 slots per row)
+#endif
+
 // (the leading scalar arguments repeat the fields of `p` that the first two memory reads need:
 // they are preloaded into SGPRs with the wave, the rest of `p` arrives by load meanwhile)
 template <typename T, int D>
@@ -190,15 +194,110 @@ __global__ void __launch_bounds__(256) pat_merge_kernel(const int32_t* __restric
   if (p.lse_out != nullptr && lane == 0) p.lse_out[pair] = total;
 }
 
-// Host launcher: one wave per (sequence, query head), four per workgroup.
+// Launches with up to 8 slots per row and many rows (tens of thousands: hundreds of requests x
+// 32-64 heads) are bound by the number of waves, each of which lives for one round trip: there a
+// half-wave takes a (sequence, head), 16 bytes of a partial row per lane, which halves the waves and
+// the load instructions per byte. Same arithmetic in the same order as the kernel above.
+template <typename T, int D>
+__global__ void __launch_bounds__(256) pat_merge_pairs_kernel(const int32_t* __restrict__ num_split_per_seq,
+                                                              const float* __restrict__ lse_part, const int num_slots,
+                                                              const int chunks_per_rank, const int max_split, const int batch,
+                                                              const int heads, const int kv_heads, const MergeParams p) {
+  constexpr int CPL = D / 32;   // columns per lane
+  constexpr int kSpec = 8;
+  const int lane = threadIdx.x & 63;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int slot_in_wg = (int)(threadIdx.x >> 6) * 2 + half;   // 8 rows per workgroup
+  int s, hq;
+  bool live;
+  if (kv_heads % 8 == 0) {
+    const int xcd = blockIdx.x & 7;
+    const int per_seq = heads >> 3;
+    int64_t u = (int64_t)(blockIdx.x >> 3) * 8 + slot_in_wg;
+    const int64_t n = (int64_t)batch * per_seq;
+    live = u < n;
+    if (!live) u = n - 1;          // (an idle half repeats the last row's reads and stores nothing)
+    s = (int)(u / per_seq);
+    const int local = (int)(u - (int64_t)s * per_seq);
+    const int group = heads / kv_heads;
+    hq = (xcd + 8 * (local / group)) * group + local % group;
+  } else {
+    int64_t u = (int64_t)blockIdx.x * 8 + slot_in_wg;
+    const int64_t n = (int64_t)batch * heads;
+    live = u < n;
+    if (!live) u = n - 1;
+    s = (int)(u / heads);
+    hq = (int)(u % heads);
+  }
+  const int64_t pair = (int64_t)s * heads + hq;
+  const float ninf = -__builtin_inff();
+  const float* __restrict__ lse = lse_part + pair * num_slots;
+  const float* __restrict__ op = p.o_part + pair * (int64_t)num_slots * D;
+  int ns = num_split_per_seq[s];
+  float l = (l32 < num_slots) ? lse[l32] : ninf;
+  float v[kSpec][CPL];
+#pragma unroll
+  for (int b = 0; b < kSpec; ++b) {
+    if (b < num_slots) {
+      const float* row = op + (int64_t)b * D + l32 * CPL;
+      if (CPL == 4) {
+        const float4 t = *(const float4*)row;
+        v[b][0] = t.x; v[b][1] = t.y; v[b][CPL - 2] = t.z; v[b][CPL - 1] = t.w;
+      } else {
+        const float2 t = *(const float2*)row;
+        v[b][0] = t.x; v[b][CPL - 1] = t.y;
+      }
+    }
+  }
+  ns = ns < 0 ? 0 : (ns > max_split ? max_split : ns);
+  const int nsl = ns * chunks_per_rank;
+  if (l32 >= nsl) l = ninf;
+  float mx = l;
+#pragma unroll
+  for (int off = kSpec / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  mx = __shfl(mx, half * 32);
+  float e = (l > ninf) ? __expf(l - mx) : 0.f;
+  float sum = e;
+#pragma unroll
+  for (int off = kSpec / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  sum = __shfl(sum, half * 32);
+  const float total = (sum > 0.f) ? mx + logf(sum) : ninf;
+  const float w_mine = (l > ninf) ? __expf(l - total) : 0.f;
+  float acc[CPL];
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
+#pragma unroll
+  for (int b = 0; b < kSpec; ++b) {
+    const float w = __shfl(w_mine, half * 32 + b);
+    if (b < num_slots && w > 0.f) {
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) acc[c] += w * v[b][c];
+    }
+  }
+  if (!live) return;
+  T* dst = (T*)p.out + (int64_t)s * p.o_stride_b + (int64_t)hq * p.o_stride_h + l32 * CPL;
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) dst[c] = (T)acc[c];
+  if (p.lse_out != nullptr && l32 == 0) p.lse_out[pair] = total;
+}
+
+// Host launcher: one wave per (sequence, query head), four per workgroup; a half-wave each in large launches
+// of few slots.
 hipError_t launch_merge(bool bf16, int head_dim, hipStream_t stream, const MergeParams& params) {
   const int64_t pairs = (int64_t)params.batch * params.heads;
-  // (a multiple of 8 kv heads: 8 interleaved lists of pairs, one per XCD, each rounded up to whole workgroups)
-  const int64_t wgs = params.kv_heads % 8 == 0 ? 8 * ((pairs / 8 + 3) / 4) : (pairs + 3) / 4;
-  const dim3 grid((unsigned)wgs), block(256);
   void (*fn)(const int32_t*, const float*, int, int, int, int, int, int, const MergeParams);
-  if (bf16) fn = head_dim == 64 ? pat_merge_kernel<__bf16, 64> : pat_merge_kernel<__bf16, 128>;
-  else fn = head_dim == 64 ? pat_merge_kernel<_Float16, 64> : pat_merge_kernel<_Float16, 128>;
+  int per_wg = 4;
+  if (params.num_slots <= 8 && pairs >= PAT_MERGE_PAIRS_MIN) {
+    per_wg = 8;
+    if (bf16) fn = head_dim == 64 ? pat_merge_pairs_kernel<__bf16, 64> : pat_merge_pairs_kernel<__bf16, 128>;
+    else fn = head_dim == 64 ? pat_merge_pairs_kernel<_Float16, 64> : pat_merge_pairs_kernel<_Float16, 128>;
+  } else {
+    if (bf16) fn = head_dim == 64 ? pat_merge_kernel<__bf16, 64> : pat_merge_kernel<__bf16, 128>;
+    else fn = head_dim == 64 ? pat_merge_kernel<_Float16, 64> : pat_merge_kernel<_Float16, 128>;
+  }
+  // (a multiple of 8 kv heads: 8 interleaved lists of pairs, one per XCD, each rounded up to whole workgroups)
+  const int64_t wgs = params.kv_heads % 8 == 0 ? 8 * ((pairs / 8 + per_wg - 1) / per_wg) : (pairs + per_wg - 1) / per_wg;
+  const dim3 grid((unsigned)wgs), block(256);
   hipLaunchKernelGGL(fn, grid, block, 0, stream, params.num_split_per_seq, params.lse_part, params.num_slots,
                      params.chunks_per_rank, params.max_split, params.batch, params.heads, params.kv_heads, params);
   return hipGetLastError();

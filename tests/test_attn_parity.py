@@ -169,6 +169,38 @@ def test_second_pack_schedule_on_one_tree():
     _assert_close("c3 second pack", out, lse, ref_out, ref_lse, w.dtype)
 
 
+@pytest.mark.parametrize("spec,heads,d,dtype", [("1,512_512,32", (32, 8), 64, torch.bfloat16),
+                                                 ("1,4,256_32,512,32", (64, 8), 128, torch.bfloat16),
+                                                 ("1,512_512,32", (32, 4), 128, torch.float16),
+                                                 ("1,700_512,32", (24, 3), 64, torch.float16)])
+def test_merge_of_many_rows(spec, heads, d, dtype):
+    # 16384 rows (requests x query heads) or more with a few partial slots each: the merge kernel gives a
+    # half-wave to every row there; both head_dims, both types, kv heads in and out of step with the 8
+    # XCDs, a row count that leaves the last workgroup part idle
+    print(f"[case] merge of many rows: {spec} heads {heads} d {d} {dtype}", flush=True)
+    import random
+    from pat_amd import generate_tree_seqs
+    dev = _device()
+    random.seed(3)
+    group, nblk = generate_tree_seqs(spec, 32)
+    w = workloads.Workload(spec, heads[0], heads[1], d, dtype, 32, group.seqlens, group.get_block_ids(), nblk, 0, 6)
+    assert w.batch * w.heads >= 16384
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    assert info.whole_sequence_tables() is None and info.max_split_per_seq >= 2
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    assert info._launch_workspace_bytes[0] > 0          # partial rows: the merge kernel ran
+    ref_out, ref_lse = _oracle(w, q, k, v)
+    _assert_close("many rows " + spec, out, lse, ref_out, ref_lse, dtype)
+
+
 def test_merge_of_more_than_256_slots(tuning):
     # five nested nodes -> every request sits in five boxes (naive_schedule: one box per node); with
     # 32-token chunks the 2048-token root reserves 64 slots per box: 320 slots per row, so the
