@@ -508,7 +508,8 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D, TALLK)) pat_split
     int f_page = 0, f_slot = 0;
     unsigned f_koff = 0, f_voff = 0;
     const unsigned ksp32 = (unsigned)ksp, vsp32 = (unsigned)vsp, k16 = (unsigned)(16 * kss), v16 = (unsigned)(16 * vss);
-    const bool fast_route = ksp == vsp && kss == vss && hpp == 1;
+    // (pages of 32, 64 or 128 tokens take the same route with the half's place inside its page added)
+    const int fast_route = (ksp == vsp && kss == vss) ? (hpp == 1 ? 1 : (hshift > 0 ? 2 : 0)) : 0;
     const int64_t kv_delta = vbase - kbase;
     auto next_half = [&]() {
       ++f_slot; f_koff += k16; f_voff += v16;
@@ -519,7 +520,7 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D, TALLK)) pat_split
     if (wave_half) next_half();
     auto fetch = [&](auto fast, int ss, u32x4 (&kd)[NP2], u32x4 (&vd)[NP2]) {
       if ((ss + 1) * SST <= ntok_u) {
-        if (decltype(fast)::value) {
+        if (decltype(fast)::value == 1) {
           const int h0 = ss * (SST / 16) + wave_half;         // this wave's first half (= page) of the super-step
           const int pgsel = h0 < 64 ? pg0 : pg1;              // (a super-step's 4 pages lie in one register)
           // (kept out of loop-invariant hoisting: next to the scalar base the 32-bit offset becomes the
@@ -530,6 +531,19 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D, TALLK)) pat_split
           for (int i = 0; i < NP2; ++i) {
             const unsigned pg = (unsigned)__builtin_amdgcn_readlane(pgsel, (h0 + i * (TPR / 16)) & 63);
             const char* ka = kbase + (uint64_t)pg * ksp32;
+            kd[i] = *(const u32x4*)(ka + ko);
+            vd[i] = *(const u32x4*)(ka + kv_delta + vo);
+          }
+        } else if (decltype(fast)::value == 2) {
+          const int h0 = ss * (SST / 16) + wave_half;         // this wave's first half of the super-step
+          const int pgsel = (h0 >> hshift) < 64 ? pg0 : pg1;  // (a super-step's pages lie in one register)
+          unsigned ko = koff, vo = voff;
+          asm volatile("" : "+v"(ko), "+v"(vo));
+#pragma unroll
+          for (int i = 0; i < NP2; ++i) {
+            const int hh = h0 + i * (TPR / 16);
+            const unsigned pg = (unsigned)__builtin_amdgcn_readlane(pgsel, (hh >> hshift) & 63);
+            const char* ka = kbase + ((uint64_t)pg * ksp32 + (unsigned)(hh & (hpp - 1)) * k16);
             kd[i] = *(const u32x4*)(ka + ko);
             vd[i] = *(const u32x4*)(ka + kv_delta + vo);
           }
@@ -657,7 +671,9 @@ __global__ void __launch_bounds__(kThreads, split_occupancy(D, TALLK)) pat_split
         }
       }
     };
-    if (fast_route) walk(std::true_type{}); else walk(std::false_type{});
+    if (fast_route == 1) walk(std::integral_constant<int, 1>{});
+    else if (fast_route == 2) walk(std::integral_constant<int, 2>{});
+    else walk(std::integral_constant<int, 0>{});
     // ---- the two wave pairs' states of the same rows are combined through LDS ----------------
     l_run = sum_xor32(l_run);
     float* xbuf = (float*)smem;                 // [rt][DB2 * 4 pieces][64 lanes] x 16 bytes
