@@ -630,6 +630,11 @@ int whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page
   int64_t total = 0, longest = 0;
   for (int32_t n : lens) { total += n; longest = std::max<int64_t>(longest, n); }
   if (longest <= 0) return 0;
+  // PAT_WHOLE_SEQUENCES=0 / 1: always the plan / always one work item per request (measurements, tests)
+  if (const char* e = std::getenv("PAT_WHOLE_SEQUENCES")) {
+    if (e[0] == '0') return 0;
+    if (e[0] == '1') return INT32_MAX;
+  }
   const int64_t token_bytes = (int64_t)kv_heads * 128 * 2 * 2;   // (at head_dim 128; the planner does not know it)
   int small = 0;
   if (longest <= whole_sequence_limit(hratio) && (int64_t)lens.size() * kv_heads <= 512 && total * token_bytes <= (int64_t)64 << 20)

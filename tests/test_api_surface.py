@@ -217,3 +217,18 @@ def test_one_work_item_per_request_where_sharing_saves_little():
     # no request in two boxes: the plan has nothing to merge either, and is launched as it is
     info, _, _ = _packed("600_64", 32, 8)
     assert info.max_split_per_seq == 1 and info.whole_sequence_tables() is None
+
+
+def test_launch_choice_can_be_forced(monkeypatch):
+    """PAT_WHOLE_SEQUENCES, read when a plan is packed: 0 keeps every batch on the plan, 1 gives every batch
+    the one-work-item-per-request tables."""
+    monkeypatch.setenv("PAT_WHOLE_SEQUENCES", "0")
+    info, _, _ = _packed("1,8_256,32", 8, 8)                 # a small batch: one item per request when left alone
+    assert info.whole_sequence_tables() is None
+    monkeypatch.setenv("PAT_WHOLE_SEQUENCES", "1")
+    info, lens, _ = _packed("1,64_2048,256", 32, 8)          # heavy sharing: the plan when left alone
+    whole = info.whole_sequence_tables()
+    assert whole is not None and whole["kv_in_CTAs"][0].tolist() == lens
+    monkeypatch.delenv("PAT_WHOLE_SEQUENCES")
+    assert _packed("1,8_256,32", 8, 8)[0].whole_sequence_tables() is not None
+    assert _packed("1,64_2048,256", 32, 8)[0].whole_sequence_tables() is None
