@@ -612,20 +612,23 @@ int whole_sequence_limit(int hratio) { return hratio >= 2 ? 768 : 384; }
 // once per request, minus U), rows = batch x query heads:
 //     one item per request  6.5 + 1.9 [a second kernel: see below] + 0.165 U + 0.070 S
 //     the plan              9.4 + 0.179 U + 0.002 S x (query heads per kv head) + 0.39 rows / 1000
+//                           (+ 0.4 rows / 1000 for every box of a request beyond two: the partial rows of
+//                           deeper trees, from 72 trees of 2-4 levels timed afterwards)
 // (mean error 6 % and 10 %). One item per request is launched when its estimate is the lower one (with the
 // plan's constant at 9.8: that decides more of the close cases right) and S is below 200 MB (the measured
 // range of close calls; beyond it the plan won every case). Over the 356 measured cases the choice is
 // within 3 % of the faster launch in 329 (always the plan: 274) and at worst 19 % slower (always the plan:
-// 66 %); e.g. plan / one item per request: 64 x (256 + 32) tokens at 64/8
+// 66 %); on the 72 deeper trees (not used for the fit) and the reference's sweep, 141 of 144 and 5 % at worst; e.g. plan / one item per request: 64 x (256 + 32) tokens at 64/8
 // heads 13.4 / 10.8 us, 8 x (1024 + 1024) at 32/8 16.6 / 14.6, 128 x (256 + 32) at 16/2 13.0 / 7.9, against
 // 128 x (256 + 32) at 32/8 15.2 / 17.9, 4 x (4096 + 32) 13.3 / 15.3. No tree of the reference's sweep changes.
 // A request walked by one workgroup needs no second kernel: up to 512 tokens, or up to 2048 when the batch
 // has a box per CU (requests x kv heads >= 256); the launch cuts longer ones into pieces and merges them.
 constexpr double kWholeSavedMaxMB = 200.;
 // Returns the longest request the one-item-per-request launch stays right for (0: launch the plan).
-// unique_tokens: tokens held by the tree's nodes; shared: some request sits in two boxes of the plan.
+// unique_tokens: tokens held by the tree's nodes; max_split: the most boxes of the plan a request sits in.
 int whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page, int hratio, int64_t unique_tokens,
-                        bool shared) {
+                        int max_split) {
+  const bool shared = max_split > 1;
   if (lens.empty() || kv_heads <= 0 || page <= 0) return 0;
   int64_t total = 0, longest = 0;
   for (int32_t n : lens) { total += n; longest = std::max<int64_t>(longest, n); }
@@ -644,7 +647,7 @@ int whole_sequences_pay(const std::vector<int32_t>& lens, int kv_heads, int page
   const double saved_mb = (double)((total - unique_tokens) * token_bytes) / 1e6;
   if (saved_mb >= kWholeSavedMaxMB) return small;
   const double rows = (double)lens.size() * kv_heads * hratio;
-  const double plan_us = 9.8 + 0.179 * unique_mb + 0.002 * saved_mb * hratio + 0.39 * rows / 1000.;
+  const double plan_us = 9.8 + 0.179 * unique_mb + 0.002 * saved_mb * hratio + (0.39 + 0.4 * std::max(0, max_split - 2)) * rows / 1000.;
   const double whole_us = 6.5 + 0.165 * unique_mb + 0.070 * saved_mb;
   if (whole_us + 1.9 < plan_us) return INT32_MAX;
   const int64_t one_kernel = (int64_t)lens.size() * kv_heads >= 256 ? 2048 : 512;
@@ -813,7 +816,7 @@ struct PrefixTreeCPP {
           pat_node_view node;
           if (pat_tree_node(native->h, i, &node) == PAT_OK && node.parent >= -1) unique += node.num_tokens;
         }
-        ws_allowed = whole_sequences_pay(batch_lens, kv_head, block_size, hratio, unique, fresh->layout.max_split_per_seq > 1);
+        ws_allowed = whole_sequences_pay(batch_lens, kv_head, block_size, hratio, unique, fresh->layout.max_split_per_seq);
       }
       if (ws_allowed > 0) {
         int64_t longest = 0;
