@@ -618,7 +618,7 @@ int whole_sequence_limit(int hratio) { return hratio >= 2 ? 768 : 384; }
 // plan's constant at 9.8: that decides more of the close cases right) and S is below 200 MB (the measured
 // range of close calls; beyond it the plan won every case). Over the 356 measured cases the choice is
 // within 3 % of the faster launch in 329 (always the plan: 274) and at worst 19 % slower (always the plan:
-// 66 %); on the 72 deeper trees (not used for the fit) and the reference's sweep, 141 of 144 and 5 % at worst; e.g. plan / one item per request: 64 x (256 + 32) tokens at 64/8
+// 66 %); on the 72 deeper trees (not used for the fit) and the reference's sweep, 141 of 144 and 4.5 % at worst; e.g. plan / one item per request: 64 x (256 + 32) tokens at 64/8
 // heads 13.4 / 10.8 us, 8 x (1024 + 1024) at 32/8 16.6 / 14.6, 128 x (256 + 32) at 16/2 13.0 / 7.9, against
 // 128 x (256 + 32) at 32/8 15.2 / 17.9, 4 x (4096 + 32) 13.3 / 15.3. No tree of the reference's sweep changes.
 // A request walked by one workgroup needs no second kernel: up to 512 tokens, or up to 2048 when the batch
