@@ -1174,6 +1174,35 @@ def test_small_batch_is_launched_as_whole_sequences():
     assert t2.kernel_info.whole_sequence_tables() is None
 
 
+@pytest.mark.parametrize("route", ["0", "1"])
+def test_request_without_tokens(route, monkeypatch):
+    # a request of length 0 beside requests that share a prefix: its rows come out as zeros with LSE -inf
+    # on both launches of the tree form (the plan, where it sits in no box and the merge kernel fills its
+    # rows; one work item per request, where its item has no tokens), the others equal the oracle
+    print(f"[case] a request without tokens, PAT_WHOLE_SEQUENCES={route}", flush=True)
+    monkeypatch.setenv("PAT_WHOLE_SEQUENCES", route)
+    dev = _device()
+    shared = list(range(1, 9))
+    rows = [[0]] + [shared + [9 + 2 * i, 10 + 2 * i] for i in range(6)]
+    lens = [0] + [16 * 10 - 3 * i for i in range(6)]
+    w = workloads.Workload("empty-request", 16, 4, 128, torch.float16, 16, lens, rows, 24, 0, 2)
+    q, k, v = w.tensors(dev)
+    tree = PrefixTreeCPP(w.page_size)
+    tree.build_radix_tree(w.seq_lens, w.padded_table())
+    tree.pack_schedule(None, w.heads // w.kv_heads, w.kv_heads)
+    info = tree.kernel_info
+    info.to_gpu(dev)
+    assert (info.whole_sequence_tables() is not None) == (route == "1")
+    assert info.num_split_per_seq.tolist()[0] == 0 and info.max_split_per_seq >= 2
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((w.batch, w.heads), float("nan"), dtype=torch.float32, device=dev)
+    prefix_attn_with_kvcache(q, k, v, tree, 1.0 / math.sqrt(w.head_dim), out, softmax_lse=lse)
+    torch.cuda.synchronize()
+    assert (out[0] == 0).all() and (lse[0] == float("-inf")).all()
+    ref_out, ref_lse = ao.paged_attention_ref(q[1:].cpu(), k.cpu(), v.cpu(), rows[1:], lens[1:])
+    _assert_close("requests beside an empty one", out[1:], lse[1:], ref_out, ref_lse, w.dtype)
+
+
 @pytest.mark.parametrize("spec,heads,kernels", [("1,8_1024,1024", (32, 8), 2), ("1,64_256,32", (64, 8), 1),
                                                 ("1,128_256,32", (16, 2), 1), ("1,4,8_512,256,704", (32, 8), 2)])
 def test_little_sharing_is_launched_as_whole_sequences(spec, heads, kernels):
